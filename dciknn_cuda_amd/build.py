@@ -1,0 +1,51 @@
+"""Compiles the gfx950 engine into dciknn_cuda_amd/libdci_hip.so with hipcc.
+
+Usage: python -m dciknn_cuda_amd.build   (cross-compiles; no GPU needed)
+"""
+import os
+import subprocess
+import sys
+from concurrent.futures import ThreadPoolExecutor
+
+HERE = os.path.dirname(os.path.abspath(__file__))
+CSRC = os.path.join(HERE, "csrc")
+LIB = os.path.join(HERE, "libdci_hip.so")
+SOURCES = ["api.hip", "project.hip", "segsort.hip", "query.hip"]
+HIPCC = os.environ.get("HIPCC", "/opt/rocm/bin/hipcc")
+FLAGS = [
+    "-O3", "-std=c++17", "-fPIC", "--offload-arch=gfx950",
+    # packed fp32 VALU ops are not to be generated on these machines
+    "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
+    "-Wall", "-Wno-unused-function",
+]
+
+
+def _compile(src):
+    obj = os.path.join(CSRC, os.path.splitext(src)[0] + ".o")
+    cmd = [HIPCC] + FLAGS + ["-c", os.path.join(CSRC, src), "-o", obj]
+    r = subprocess.run(cmd, capture_output=True, text=True)
+    return src, obj, r
+
+
+def build_library(verbose=False):
+    """(Re)compile every source and link the shared library; returns its path."""
+    with ThreadPoolExecutor(max_workers=4) as ex:
+        results = list(ex.map(_compile, SOURCES))
+    objs = []
+    for src, obj, r in results:
+        noise = "\n".join(l for l in r.stderr.splitlines()
+                          if "packed-fp32-ops" not in l)
+        if r.returncode != 0:
+            raise RuntimeError("hipcc failed on %s:\n%s" % (src, r.stderr))
+        if verbose and noise.strip():
+            print(noise, file=sys.stderr)
+        objs.append(obj)
+    cmd = [HIPCC, "-shared", "-fPIC", "--offload-arch=gfx950", "-o", LIB] + objs
+    r = subprocess.run(cmd, capture_output=True, text=True)
+    if r.returncode != 0:
+        raise RuntimeError("link failed:\n%s" % r.stderr)
+    return LIB
+
+
+if __name__ == "__main__":
+    print(build_library(verbose=True))

@@ -1,0 +1,212 @@
+"""Python interface of the MI355X Prioritized DCI engine.
+
+`DCI` and `MDCI` keep the public behaviour of the reference's
+dciknn_cuda/core.py:25-169 (argument names, defaults, exception types, return
+shapes and dtypes) on top of libdci_hip.so.  Additions, all keyword-only and
+optional: `seed` / `directions` at construction and the `directions` property
+(the reference can neither seed, inject nor read its directions), and
+`return_int` / `return_counters` on `query`.
+"""
+import torch
+
+from . import _capi
+
+
+def _stream_ptr(device):
+    return torch.cuda.current_stream(device).cuda_stream
+
+
+class DCI(object):
+
+    def __init__(self, dim, num_comp_indices=2, num_simp_indices=7, bs=100, ts=10, device=0,
+                 *, seed=0, directions=None):
+        if not torch.cuda.is_available():
+            raise RuntimeError("DCI requires GPU access, please check the ROCm driver.")
+        self._dim = dim
+        self._num_comp_indices = num_comp_indices
+        self._num_simp_indices = num_simp_indices
+        self._device = torch.device("cuda", device if isinstance(device, int) else
+                                    torch.device(device).index or 0)
+        self._lib = _capi.lib()
+        handle = _capi.ctypes.c_void_p()
+        _capi.check(self._lib.dcih_create(dim, num_comp_indices, num_simp_indices,
+                                          self._device.index, seed,
+                                          _capi.ctypes.byref(handle)))
+        self._dci_inst = handle
+        self._array = None
+        self._block_size = bs
+        self._thread_size = ts
+        self.num_points = 0
+        if directions is not None:
+            self.directions = directions
+
+    def __del__(self):
+        try:
+            self.free()
+        except Exception:
+            pass
+
+    @property
+    def dim(self):
+        return self._dim
+
+    @property
+    def num_comp_indices(self):
+        return self._num_comp_indices
+
+    @property
+    def num_simp_indices(self):
+        return self._num_simp_indices
+
+    @property
+    def directions(self):
+        """The unit projection directions, a CPU float32 tensor [m*L, dim]."""
+        self._require_handle()
+        out = torch.empty(self._num_comp_indices * self._num_simp_indices, self._dim,
+                          dtype=torch.float32)
+        _capi.check(self._lib.dcih_get_directions(self._dci_inst, out.data_ptr()))
+        return out
+
+    @directions.setter
+    def directions(self, value):
+        self._require_handle()
+        value = torch.as_tensor(value, dtype=torch.float32).cpu().contiguous()
+        want = (self._num_comp_indices * self._num_simp_indices, self._dim)
+        if tuple(value.shape) != want:
+            raise ValueError("directions must have shape %s" % (want,))
+        _capi.check(self._lib.dcih_set_directions(self._dci_inst, value.data_ptr()))
+
+    def _require_handle(self):
+        if self._dci_inst is None:
+            raise RuntimeError("this DCI instance has been freed")
+
+    def _ensure_positive_integer(self, x):
+        if not isinstance(x, int):
+            raise TypeError("number must be an integer")
+        elif x <= 0:
+            raise ValueError("number must be positive")
+
+    def _check_data(self, arr):
+        if arr.shape[1] != self.dim:
+            raise ValueError("mismatch between tensor dimension (%d) and the declared dimension of this DCI instance (%d)" % (arr.shape[1], self.dim))
+        if arr.dtype != torch.float:
+            raise TypeError("tensor must consist of single-precision floats")
+        if not arr.is_contiguous():
+            raise ValueError("the memory layout of tensor must be in row-major (C-order)")
+        if not arr.is_cuda:
+            raise TypeError("tensor must be a cuda tensor")
+
+    def add(self, data):
+        self._require_handle()
+        if self.num_points > 0:
+            raise RuntimeError("DCI class does not support insertion of more than one tensor. Must combine all tensors into one tensor before inserting")
+        self._check_data(data)
+        if data.device != self._device:
+            raise ValueError("tensor is on %s but this DCI instance lives on %s" % (data.device, self._device))
+        _capi.check(self._lib.dcih_add(self._dci_inst, self._dim, data.shape[0], data.data_ptr(),
+                                       self._block_size, self._thread_size,
+                                       _stream_ptr(self._device)))
+        self.num_points = data.shape[0]
+        self._array = data   # the index borrows this memory
+
+    # query is num_queries x dim, returns num_queries x num_neighbours
+    def query(self, query, num_neighbours=-1, num_outer_iterations=5000, blind=False,
+              *, return_int=False, return_counters=False):
+        self._require_handle()
+        if len(query.shape) < 2:
+            _query = query.unsqueeze(0)
+        else:
+            _query = query
+        self._check_data(_query)
+        if num_neighbours < 0:
+            num_neighbours = self.num_points
+        self._ensure_positive_integer(num_neighbours)
+        if blind:
+            raise NotImplementedError("blind querying is not available in this build")
+        if self.num_points == 0:
+            raise RuntimeError("query on an empty DCI instance; call add() first")
+        if num_neighbours > self.num_points:
+            raise ValueError("num_neighbours exceeds the number of indexed points")
+        max_num_candidates = 10 * num_neighbours
+        nq = _query.shape[0]
+        ids = torch.empty((nq, num_neighbours), dtype=torch.int32, device=self._device)
+        dists = torch.empty((nq, num_neighbours), dtype=torch.float32, device=self._device)
+        counters = None
+        if return_counters:
+            counters = torch.empty((nq, _capi.NUM_COUNTERS), dtype=torch.int64, device=self._device)
+        _capi.check(self._lib.dcih_query(
+            self._dci_inst, self._dim, nq, _query.data_ptr(), num_neighbours, 0,
+            num_outer_iterations, max_num_candidates, self._block_size, self._thread_size,
+            ids.data_ptr(), dists.data_ptr(),
+            counters.data_ptr() if counters is not None else None,
+            _stream_ptr(self._device)))
+        if not return_int:
+            ids = ids.to(torch.float32)   # the reference returns ids as floats
+        if return_counters:
+            return ids, dists, counters
+        return ids, dists
+
+    def clear(self):
+        self._require_handle()
+        _capi.check(self._lib.dcih_clear(self._dci_inst))
+        self.num_points = 0
+        self._array = None
+
+    def reset(self):
+        self._require_handle()
+        _capi.check(self._lib.dcih_reset(self._dci_inst))
+        self.num_points = 0
+        self._array = None
+
+    def free(self):
+        if getattr(self, "_dci_inst", None) is not None:
+            self._lib.dcih_free(self._dci_inst)
+            self._dci_inst = None
+        self.num_points = 0
+        self._array = None
+
+
+class MDCI(object):
+    """Multi-device front end of the reference, accepted with one device only."""
+
+    def __init__(self, dim, num_comp_indices=2, num_simp_indices=7, bs=100, ts=10, devices=[0],
+                 **kwargs):
+        devices = list(devices)
+        if len(devices) != 1:
+            raise NotImplementedError(
+                "this build runs on one GPU: pass devices=[<one device id>]")
+        self.devices = devices
+        self.num_devices = 1
+        self.dcis = [DCI(dim, num_comp_indices, num_simp_indices, bs, ts, dev, **kwargs)
+                     for dev in devices]
+        self.data_per_device = 0
+
+    def add(self, data):
+        self.data_per_device = data.shape[0] // self.num_devices + 1
+        cur_data = data[0:self.data_per_device].to(self.dcis[0]._device)
+        self.dcis[0].add(cur_data)
+
+    def query(self, query, num_neighbours=-1, num_outer_iterations=5000, blind=False):
+        if num_neighbours <= 0:
+            raise RuntimeError('num_neighbours must be positive')
+        if len(query.shape) < 2:
+            _query = query.unsqueeze(0)
+        else:
+            _query = query
+        _query = _query.detach().clone().to(self.dcis[0]._device)
+        nns, dists = self.dcis[0].query(_query, num_neighbours, num_outer_iterations, blind)
+        _, sort_indices = torch.sort(dists, dim=1, stable=True)
+        sort_indices = sort_indices[:, :num_neighbours]
+        return torch.gather(nns, 1, sort_indices), torch.gather(dists, 1, sort_indices)
+
+    def clear(self):
+        for dci in self.dcis:
+            dci.clear()
+
+    def reset(self):
+        for dci in self.dcis:
+            dci.reset()
+
+    def free(self):
+        for dci in self.dcis:
+            dci.free()

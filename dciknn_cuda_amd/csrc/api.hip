@@ -1,0 +1,341 @@
+// Host side of libdci_hip.so: the C-ABI declared in include/dci_hip.h.
+//
+// Mirrors the host functions of the reference (dci_init, dci_add, dci_query,
+// dci_clear, dci_reset, dci_free: src/dci_cuda_kernel.cu:77-187, :777-899) but
+// returns status codes instead of asserting, takes a stream, frees what it
+// allocates, and launches a constant number of kernels per call instead of
+// several per query.
+#include <cmath>
+#include <cstring>
+#include <new>
+#include <string>
+#include <vector>
+
+#include "../../include/dci_hip.h"
+#include "common.h"
+#include "kernels.h"
+
+namespace dcih {
+
+static thread_local std::string g_last_error;
+
+int fail(int code, const std::string& msg) {
+    g_last_error = msg;
+    return code;
+}
+
+namespace {
+
+// splitmix64 -> xoshiro256** -> Box-Muller in double: the same seed gives the
+// same directions on every machine.
+struct Rng {
+    uint64_t s[4];
+    bool have_spare = false;
+    double spare = 0.0;
+    explicit Rng(uint64_t seed) {
+        uint64_t x = seed;
+        for (int i = 0; i < 4; i++) {
+            x += 0x9e3779b97f4a7c15ull;
+            uint64_t z = x;
+            z = (z ^ (z >> 30)) * 0xbf58476d1ce4e5b9ull;
+            z = (z ^ (z >> 27)) * 0x94d049bb133111ebull;
+            s[i] = z ^ (z >> 31);
+        }
+    }
+    static uint64_t rotl(uint64_t v, int k) { return (v << k) | (v >> (64 - k)); }
+    uint64_t next() {
+        const uint64_t r = rotl(s[1] * 5, 7) * 9;
+        const uint64_t t = s[1] << 17;
+        s[2] ^= s[0]; s[3] ^= s[1]; s[1] ^= s[2]; s[0] ^= s[3];
+        s[2] ^= t; s[3] = rotl(s[3], 45);
+        return r;
+    }
+    double uniform() { return ((next() >> 11) + 0.5) * (1.0 / 9007199254740992.0); }  // (0,1)
+    double normal() {
+        if (have_spare) { have_spare = false; return spare; }
+        const double u = uniform(), v = uniform();
+        const double r = std::sqrt(-2.0 * std::log(u));
+        const double th = 6.283185307179586476925 * v;
+        spare = r * std::sin(th);
+        have_spare = true;
+        return r * std::cos(th);
+    }
+};
+
+struct DeviceGuard {
+    int prev = -1;
+    bool ok;
+    explicit DeviceGuard(int dev) {
+        ok = hipGetDevice(&prev) == hipSuccess && hipSetDevice(dev) == hipSuccess;
+    }
+    ~DeviceGuard() { if (prev >= 0) (void)hipSetDevice(prev); }
+};
+
+}  // namespace
+}  // namespace dcih
+
+using namespace dcih;
+
+struct dcih_index {
+    int dim = 0, M = 0, L = 0, device = 0;
+    uint64_t seed = 0;
+    uint64_t draws = 0;                 // direction sets drawn so far
+    std::vector<float> h_dirs;          // [I][dim]
+    float* d_dirs = nullptr;
+    const float* d_data = nullptr;      // borrowed
+    int64_t n = 0;
+    int block_size = 0;
+    float* d_skeys = nullptr;           // [I][n]
+    int32_t* d_sids = nullptr;          // [I][n]
+    // grow-only query workspace
+    void* ws = nullptr;
+    size_t ws_bytes = 0;
+};
+
+namespace {
+
+int num_indices(const dcih_index* h) { return h->M * h->L; }
+
+// Draws direction set number h->draws from the handle's seed and uploads it.
+int draw_directions(dcih_index* h) {
+    const int I = num_indices(h);
+    Rng rng(h->seed + 0x632be59bd9b4e019ull * h->draws);
+    h->draws++;
+    h->h_dirs.resize((size_t)I * h->dim);
+    for (auto& v : h->h_dirs) v = (float)rng.normal();
+    // unit rows: sequential fp32 sum of squares, sqrtf, divide
+    // (normalize_proj_vecs, src/dci_cuda_kernel.cu:52-73)
+    for (int r = 0; r < I; r++) {
+        float* row = h->h_dirs.data() + (size_t)r * h->dim;
+        float sq = 0.0f;
+        for (int k = 0; k < h->dim; k++) sq += row[k] * row[k];
+        const float norm = sqrtf(sq);
+        for (int k = 0; k < h->dim; k++) row[k] /= norm;
+    }
+    DCIH_HIP(hipMemcpy(h->d_dirs, h->h_dirs.data(), h->h_dirs.size() * sizeof(float),
+                       hipMemcpyHostToDevice));
+    return 0;
+}
+
+int release_index(dcih_index* h) {
+    if (h->d_skeys) { DCIH_HIP(hipFree(h->d_skeys)); h->d_skeys = nullptr; }
+    if (h->d_sids) { DCIH_HIP(hipFree(h->d_sids)); h->d_sids = nullptr; }
+    h->d_data = nullptr;
+    h->n = 0;
+    h->block_size = 0;
+    return 0;
+}
+
+int ensure_ws(dcih_index* h, size_t bytes) {
+    if (bytes <= h->ws_bytes) return 0;
+    if (h->ws) { DCIH_HIP(hipFree(h->ws)); h->ws = nullptr; h->ws_bytes = 0; }
+    DCIH_HIP(hipMalloc(&h->ws, bytes));
+    h->ws_bytes = bytes;
+    return 0;
+}
+
+size_t align_up(size_t v) { return (v + 255) & ~(size_t)255; }
+
+}  // namespace
+
+extern "C" {
+
+const char* dcih_last_error(void) { return g_last_error.c_str(); }
+
+int dcih_abi_version(void) { return 1; }
+
+int dcih_create(int dim, int num_comp_indices, int num_simp_indices, int device,
+                uint64_t seed, dcih_index** out) {
+    if (!out) return fail(DCIH_EINVAL, "dcih_create: out is null");
+    *out = nullptr;
+    if (dim <= 0 || num_comp_indices <= 0 || num_simp_indices <= 0)
+        return fail(DCIH_EINVAL, "dcih_create: dim and index counts must be positive");
+    if ((int64_t)num_comp_indices * num_simp_indices > (1 << 20))
+        return fail(DCIH_EINVAL, "dcih_create: too many simple indices");
+    int ndev = 0;
+    DCIH_HIP(hipGetDeviceCount(&ndev));
+    if (device < 0 || device >= ndev) return fail(DCIH_EINVAL, "dcih_create: no such device");
+    DeviceGuard guard(device);
+    if (!guard.ok) return fail(DCIH_EHIP, "dcih_create: cannot select device");
+    dcih_index* h = new (std::nothrow) dcih_index();
+    if (!h) return fail(DCIH_EHIP, "dcih_create: out of host memory");
+    h->dim = dim; h->M = num_comp_indices; h->L = num_simp_indices;
+    h->device = device; h->seed = seed;
+    const size_t bytes = (size_t)num_indices(h) * dim * sizeof(float);
+    if (hipMalloc(&h->d_dirs, bytes) != hipSuccess) {
+        delete h;
+        return fail(DCIH_EHIP, "dcih_create: hipMalloc of the directions failed");
+    }
+    const int rc = draw_directions(h);
+    if (rc) { (void)hipFree(h->d_dirs); delete h; return rc; }
+    *out = h;
+    return DCIH_OK;
+}
+
+int dcih_get_directions(const dcih_index* h, float* h_dirs) {
+    if (!h || !h_dirs) return fail(DCIH_EINVAL, "dcih_get_directions: null argument");
+    std::memcpy(h_dirs, h->h_dirs.data(), h->h_dirs.size() * sizeof(float));
+    return DCIH_OK;
+}
+
+int dcih_set_directions(dcih_index* h, const float* h_dirs) {
+    if (!h || !h_dirs) return fail(DCIH_EINVAL, "dcih_set_directions: null argument");
+    if (h->n > 0) return fail(DCIH_ESTATE, "dcih_set_directions: index is not empty");
+    DeviceGuard guard(h->device);
+    std::memcpy(h->h_dirs.data(), h_dirs, h->h_dirs.size() * sizeof(float));
+    DCIH_HIP(hipMemcpy(h->d_dirs, h_dirs, h->h_dirs.size() * sizeof(float), hipMemcpyHostToDevice));
+    return DCIH_OK;
+}
+
+int dcih_add(dcih_index* h, int dim, int64_t num_points, const float* d_data,
+             int block_size, int thread_size, void* stream) {
+    if (!h) return fail(DCIH_EINVAL, "dcih_add: null handle");
+    if (dim != h->dim) return fail(DCIH_EINVAL, "dcih_add: dim differs from the index's");
+    if (h->n > 0) return fail(DCIH_ESTATE, "dcih_add: index already holds points; clear it first");
+    if (num_points <= 0 || !d_data) return fail(DCIH_EINVAL, "dcih_add: no points given");
+    if (num_points > 0x7fffffffLL) return fail(DCIH_EINVAL, "dcih_add: more than 2^31-1 points");
+    if (block_size <= 0 || thread_size <= 0)
+        return fail(DCIH_EINVAL, "dcih_add: block_size and thread_size must be positive");
+    DeviceGuard guard(h->device);
+    hipStream_t s = (hipStream_t)stream;
+    const int I = num_indices(h);
+    const size_t cells = (size_t)I * num_points;
+    float* d_keys = nullptr;
+    void* d_tmp = nullptr;
+    const size_t tmp_bytes = segsort_tmp_bytes(I, num_points, block_size);
+    int rc = DCIH_OK;
+    do {
+        if (hipMalloc(&h->d_skeys, cells * sizeof(float)) != hipSuccess ||
+            hipMalloc(&h->d_sids, cells * sizeof(int32_t)) != hipSuccess ||
+            hipMalloc(&d_keys, cells * sizeof(float)) != hipSuccess ||
+            (tmp_bytes && hipMalloc(&d_tmp, tmp_bytes) != hipSuccess)) {
+            rc = fail(DCIH_EHIP, "dcih_add: out of device memory");
+            break;
+        }
+        rc = project(h->d_dirs, I, d_data, num_points, dim, d_keys, s);
+        if (rc) break;
+        rc = segsort(d_keys, I, num_points, block_size, h->d_skeys, h->d_sids, d_tmp, s);
+    } while (0);
+    // the scratch buffers are in use until the stream drains
+    const hipError_t se = hipStreamSynchronize(s);
+    if (d_keys) (void)hipFree(d_keys);
+    if (d_tmp) (void)hipFree(d_tmp);
+    if (rc == DCIH_OK && se != hipSuccess)
+        rc = fail(DCIH_EHIP, std::string("dcih_add: ") + hipGetErrorString(se));
+    if (rc) { (void)release_index(h); return rc; }
+    h->d_data = d_data;
+    h->n = num_points;
+    h->block_size = block_size;
+    return DCIH_OK;
+}
+
+int dcih_query(dcih_index* h, int dim, int num_queries, const float* d_query,
+               int num_neighbours, int blind, int num_outer_iterations,
+               int max_num_candidates, int block_size, int thread_size,
+               int32_t* d_nn, float* d_dists, uint64_t* d_counters, void* stream) {
+    if (!h) return fail(DCIH_EINVAL, "dcih_query: null handle");
+    if (blind) return fail(DCIH_EUNSUPPORTED, "dcih_query: blind querying is not built");
+    if (dim != h->dim) return fail(DCIH_EINVAL, "dcih_query: dim differs from the index's");
+    if (h->n <= 0) return fail(DCIH_ESTATE, "dcih_query: index is empty");
+    if (num_neighbours <= 0 || num_neighbours > h->n)
+        return fail(DCIH_EINVAL, "dcih_query: num_neighbours must be in [1, num_points]");
+    if (num_queries < 0 || (num_queries > 0 && (!d_query || !d_nn || !d_dists)))
+        return fail(DCIH_EINVAL, "dcih_query: null buffer");
+    if (thread_size <= 0) return fail(DCIH_EINVAL, "dcih_query: thread_size must be positive");
+    if (block_size != h->block_size)
+        return fail(DCIH_EINVAL, "dcih_query: block_size differs from the one the index was built with");
+    if (num_queries == 0) return DCIH_OK;
+    DeviceGuard guard(h->device);
+    hipStream_t s = (hipStream_t)stream;
+    const int I = num_indices(h);
+
+    QueryArgs a;
+    a.skeys = h->d_skeys; a.sids = h->d_sids; a.data = h->d_data; a.query = d_query;
+    a.N = h->n;
+    a.ppb = (h->n + block_size - 1) / block_size;
+    a.dim = dim; a.M = h->M; a.L = h->L; a.B = block_size; a.T = thread_size;
+    a.nq = num_queries; a.k = num_neighbours;
+    a.kcap = (int)std::min<int64_t>(num_neighbours, a.ppb);
+    a.stop_at = (int64_t)num_outer_iterations * h->L;
+    a.max_cand = max_num_candidates;
+    a.counters = (unsigned long long*)d_counters;
+    a.out_ids = d_nn; a.out_dists = d_dists;
+
+    const size_t qp_bytes = align_up((size_t)I * num_queries * sizeof(float));
+    const size_t part_bytes = align_up(query_part_bytes(a));
+    const size_t gs_bytes = align_up(query_gscratch_bytes(a));
+    int rc = ensure_ws(h, qp_bytes + part_bytes + gs_bytes);
+    if (rc) return rc;
+    char* base = (char*)h->ws;
+    float* d_qproj = (float*)base;
+    a.qproj = d_qproj;
+    a.part = (unsigned long long*)(base + qp_bytes);
+    a.gscratch = gs_bytes ? (uint32_t*)(base + qp_bytes + part_bytes) : nullptr;
+
+    rc = project(h->d_dirs, I, d_query, num_queries, dim, d_qproj, s);
+    if (rc) return rc;
+    return query(a, s);
+}
+
+int dcih_get_index(const dcih_index* h, float* h_keys, int32_t* h_ids) {
+    if (!h) return fail(DCIH_EINVAL, "dcih_get_index: null handle");
+    if (h->n <= 0) return fail(DCIH_ESTATE, "dcih_get_index: index is empty");
+    DeviceGuard guard(h->device);
+    const size_t cells = (size_t)num_indices(h) * h->n;
+    DCIH_HIP(hipDeviceSynchronize());
+    if (h_keys) DCIH_HIP(hipMemcpy(h_keys, h->d_skeys, cells * sizeof(float), hipMemcpyDeviceToHost));
+    if (h_ids) DCIH_HIP(hipMemcpy(h_ids, h->d_sids, cells * sizeof(int32_t), hipMemcpyDeviceToHost));
+    return DCIH_OK;
+}
+
+int64_t dcih_num_points(const dcih_index* h) { return h ? h->n : 0; }
+
+int dcih_clear(dcih_index* h) {
+    if (!h) return fail(DCIH_EINVAL, "dcih_clear: null handle");
+    DeviceGuard guard(h->device);
+    DCIH_HIP(hipDeviceSynchronize());
+    return release_index(h);
+}
+
+int dcih_reset(dcih_index* h) {
+    const int rc = dcih_clear(h);
+    if (rc) return rc;
+    DeviceGuard guard(h->device);
+    return draw_directions(h);
+}
+
+int dcih_free(dcih_index* h) {
+    if (!h) return DCIH_OK;
+    DeviceGuard guard(h->device);
+    (void)hipDeviceSynchronize();
+    (void)release_index(h);
+    if (h->ws) (void)hipFree(h->ws);
+    if (h->d_dirs) (void)hipFree(h->d_dirs);
+    delete h;
+    return DCIH_OK;
+}
+
+int dcih_project(const float* d_dirs, int num_idx, const float* d_rows, int64_t num_rows,
+                 int dim, float* d_out, void* stream) {
+    if (!d_dirs || !d_rows || !d_out || num_idx <= 0 || num_rows < 0 || dim <= 0)
+        return fail(DCIH_EINVAL, "dcih_project: bad argument");
+    return project(d_dirs, num_idx, d_rows, num_rows, dim, d_out, (hipStream_t)stream);
+}
+
+int dcih_segsort(const float* d_keys, int num_idx, int64_t num_points, int block_size,
+                 float* d_skeys, int32_t* d_sids, void* stream) {
+    if (!d_keys || !d_skeys || !d_sids || num_idx <= 0 || num_points <= 0 || block_size <= 0)
+        return fail(DCIH_EINVAL, "dcih_segsort: bad argument");
+    hipStream_t s = (hipStream_t)stream;
+    const size_t tmp_bytes = segsort_tmp_bytes(num_idx, num_points, block_size);
+    void* d_tmp = nullptr;
+    if (tmp_bytes) DCIH_HIP(hipMalloc(&d_tmp, tmp_bytes));
+    const int rc = segsort(d_keys, num_idx, num_points, block_size, d_skeys, d_sids, d_tmp, s);
+    if (d_tmp) {
+        (void)hipStreamSynchronize(s);
+        (void)hipFree(d_tmp);
+    }
+    return rc;
+}
+
+}  // extern "C"

@@ -1,0 +1,139 @@
+/*
+ * C-ABI of the MI355X (gfx950) Prioritized DCI engine: libdci_hip.so.
+ *
+ * Plain C types only: pointers, sizes, an opaque handle and a stream passed as
+ * void* (a hipStream_t; NULL = the default stream).  Every entry point returns
+ * 0 on success or a negative DCIH_E* code; dcih_last_error() then holds a
+ * message for the calling thread.  Device pointers are marked d_, host
+ * pointers h_.  Unless stated otherwise a call only enqueues work on `stream`;
+ * outputs are valid once the stream has been synchronised.
+ *
+ * Each entry point names the interface of the CUDA reference
+ * (niopeng/dciknn_cuda, paths relative to its root) that it stands in for.
+ */
+#ifndef DCI_HIP_H
+#define DCI_HIP_H
+
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+typedef struct dcih_index dcih_index;
+
+enum {
+    DCIH_OK = 0,
+    DCIH_EINVAL = -1,      /* bad argument (the reference would assert) */
+    DCIH_ESTATE = -2,      /* call not valid in this state, e.g. add() twice */
+    DCIH_EHIP = -3,        /* a HIP runtime call failed */
+    DCIH_EUNSUPPORTED = -4 /* valid in the reference, not built here yet */
+};
+
+/* Per-query traversal counters written by dcih_query when asked for. */
+enum {
+    DCIH_CTR_VISITED = 0,   /* in-range index entries visited            */
+    DCIH_CTR_CANDIDATES = 1,/* points promoted = exact distances computed */
+    DCIH_CTR_PROBES = 2,    /* key reads made by the positioning search   */
+    DCIH_CTR_STEPS = 3,     /* outer steps executed, summed over partitions */
+    DCIH_NUM_COUNTERS = 4
+};
+
+/* Message for the last failing call on this thread ("" if none). */
+const char* dcih_last_error(void);
+
+/* Library/ABI version, bumped on any signature change. */
+int dcih_abi_version(void);
+
+/*
+ * Replaces dci_init (include/dci.h:61, src/dci_cuda_kernel.cu:93-110) and the
+ * handle allocation in py_dci_new (src/dci_cuda.cpp:54-66).  Draws
+ * num_comp_indices*num_simp_indices N(0,1) directions of length dim on the
+ * HOST from `seed` (the reference draws them on device from an unseeded libc
+ * rand(), src/util_kernel.cu:119-137) and scales each row to unit L2 norm the
+ * way normalize_proj_vecs does (src/dci_cuda_kernel.cu:52-73).  Synchronous.
+ */
+int dcih_create(int dim, int num_comp_indices, int num_simp_indices, int device,
+                uint64_t seed, dcih_index** out);
+
+/*
+ * No counterpart in the reference (its directions can be neither read nor
+ * injected); needed so two implementations can be compared on identical
+ * directions.  h_dirs is row-major [num_comp*num_simp][dim].  `set` stores the
+ * values as given (no normalisation) and is only legal while the index is
+ * empty.  Both synchronous.
+ */
+int dcih_get_directions(const dcih_index* h, float* h_dirs);
+int dcih_set_directions(dcih_index* h, const float* h_dirs);
+
+/*
+ * Replaces dci_add (include/dci.h:68, src/dci_cuda_kernel.cu:149-187): projects
+ * num_points rows of d_data (row-major [num_points][dim], fp32) on every
+ * direction and sorts each (simple index, partition) slice, with
+ * ceil(num_points/block_size) points per partition.  Like the reference the
+ * index BORROWS d_data: it must stay valid and unchanged until dcih_clear /
+ * dcih_reset / dcih_free.  A second add on a non-empty index returns
+ * DCIH_ESTATE (the reference asserts, :157).  thread_size does not influence
+ * the result of the build and is accepted for signature parity.
+ */
+int dcih_add(dcih_index* h, int dim, int64_t num_points, const float* d_data,
+             int block_size, int thread_size, void* stream);
+
+/*
+ * Replaces dci_query (include/dci.h:71, src/dci_cuda_kernel.cu:777-875) with
+ * query_config.blind == false.  d_query is [num_queries][dim]; for each query
+ * d_nn / d_dists [num_queries][num_neighbours] receive the ids and Euclidean
+ * distances of the num_neighbours best promoted candidates, ascending by
+ * (distance, id); slots beyond the number of candidates get id -1 and +inf.
+ * block_size must equal the value given to dcih_add (the partitioning is part
+ * of the built index); thread_size is the window width.  d_counters is NULL or
+ * [num_queries][DCIH_NUM_COUNTERS].  blind != 0 returns DCIH_EUNSUPPORTED.
+ */
+int dcih_query(dcih_index* h, int dim, int num_queries, const float* d_query,
+               int num_neighbours, int blind, int num_outer_iterations,
+               int max_num_candidates, int block_size, int thread_size,
+               int32_t* d_nn, float* d_dists, uint64_t* d_counters, void* stream);
+
+/*
+ * Inspection of the built index (no counterpart in the reference besides the
+ * debug printer dci_dump, src/dci_cuda_kernel.cu:901-912).  Copies the sorted
+ * projections and point ids, both [num_indices][num_points], to host buffers;
+ * either pointer may be NULL.  Synchronous.
+ */
+int dcih_get_index(const dcih_index* h, float* h_keys, int32_t* h_ids);
+
+/* Number of points currently indexed (0 when empty). */
+int64_t dcih_num_points(const dcih_index* h);
+
+/* Replaces dci_clear (include/dci.h:77, src/dci_cuda_kernel.cu:878-885). */
+int dcih_clear(dcih_index* h);
+
+/*
+ * Replaces dci_reset (include/dci.h:80, src/dci_cuda_kernel.cu:887-891): clear,
+ * then draw fresh directions (the next draw of the handle's seeded sequence).
+ */
+int dcih_reset(dcih_index* h);
+
+/*
+ * Replaces dci_free (include/dci.h:82, src/dci_cuda_kernel.cu:893-899) plus the
+ * handle release in py_dci_free (src/dci_cuda.cpp:162-173).  NULL is a no-op.
+ */
+int dcih_free(dcih_index* h);
+
+/*
+ * Stand-alone pieces of the build, exposed so each kernel can be checked and
+ * timed on its own.  d_keys is [num_indices][num_points].
+ *   dcih_project : out[r][c] = sum_k d_rows[c][k] * d_dirs[r][k]  (the SGEMM at
+ *                  src/util_kernel.cu:76 as used at src/dci_cuda_kernel.cu:167-169)
+ *   dcih_segsort : copy_to_indices + sort_indices
+ *                  (src/dci_cuda_kernel.cu:113-146), ties by id
+ */
+int dcih_project(const float* d_dirs, int num_indices, const float* d_rows,
+                 int64_t num_rows, int dim, float* d_out, void* stream);
+int dcih_segsort(const float* d_keys, int num_indices, int64_t num_points,
+                 int block_size, float* d_skeys, int32_t* d_sids, void* stream);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* DCI_HIP_H */

@@ -1,0 +1,48 @@
+"""Helpers shared by the parity tests."""
+import numpy as np
+import torch
+
+
+def set_agreement(ids_a, ids_b):
+    """Mean fraction of each row of ids_a found in the same row of ids_b."""
+    ids_a, ids_b = np.asarray(ids_a), np.asarray(ids_b)
+    hit = 0
+    for a, b in zip(ids_a, ids_b):
+        hit += len(set(a.tolist()) & set(b.tolist()))
+    return hit / ids_a.size
+
+
+def engine_index(dci):
+    """(skeys, sids) of a built DCI instance as numpy arrays [I][N]."""
+    from dciknn_cuda_amd import _capi
+    I = dci.num_comp_indices * dci.num_simp_indices
+    keys = np.empty((I, dci.num_points), np.float32)
+    ids = np.empty((I, dci.num_points), np.int32)
+    _capi.check(dci._lib.dcih_get_index(dci._dci_inst, keys.ctypes.data, ids.ctypes.data))
+    return keys, ids
+
+
+def engine_project(dirs, rows):
+    """dcih_project on cuda:0: numpy [I][dim], [n][dim] -> numpy [I][n]."""
+    from dciknn_cuda_amd import _capi
+    d = torch.as_tensor(dirs, dtype=torch.float32).cuda().contiguous()
+    r = torch.as_tensor(rows, dtype=torch.float32).cuda().contiguous()
+    out = torch.empty((d.shape[0], r.shape[0]), dtype=torch.float32, device="cuda")
+    _capi.check(_capi.lib().dcih_project(d.data_ptr(), d.shape[0], r.data_ptr(), r.shape[0],
+                                         d.shape[1], out.data_ptr(),
+                                         torch.cuda.current_stream().cuda_stream))
+    torch.cuda.synchronize()
+    return out.cpu().numpy()
+
+
+def engine_segsort(keys, block_size):
+    """dcih_segsort on cuda:0: numpy [I][n] -> (skeys, sids) numpy."""
+    from dciknn_cuda_amd import _capi
+    k = torch.as_tensor(keys, dtype=torch.float32).cuda().contiguous()
+    sk = torch.empty_like(k)
+    si = torch.empty(k.shape, dtype=torch.int32, device="cuda")
+    _capi.check(_capi.lib().dcih_segsort(k.data_ptr(), k.shape[0], k.shape[1], block_size,
+                                         sk.data_ptr(), si.data_ptr(),
+                                         torch.cuda.current_stream().cuda_stream))
+    torch.cuda.synchronize()
+    return sk.cpu().numpy(), si.cpu().numpy()
