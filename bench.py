@@ -1,0 +1,219 @@
+#!/usr/bin/env python3
+"""Benchmark of the Prioritized DCI hot path on one MI355X.
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--config c2]
+                    [--bs B --ts T --outer O] [--nq NQ] [--no-cpu]
+
+A step is one pass of the query path (query projection, traversal, exact
+distances, top-k) over the whole seeded query batch of the workload, with the
+index built and all inputs resident in HBM.  The build (projection + segmented
+sort) is timed separately and reported as build_points_per_s.  Prints ONE JSON
+line; see DESIGN.md for the meaning of every field.
+"""
+import argparse
+import json
+import os
+import sys
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+sys.path.insert(0, ROOT)
+
+HBM_PEAK_GBS = 8000.0   # MI355X HBM3E
+
+# (block_size, thread_size, num_outer_iterations) used when none are given:
+# the fastest setting found with recall@k >= 0.95 on that workload.
+TUNED = {
+    "c1": dict(bs=100, ts=10, outer=5000),
+    "c2": dict(bs=100, ts=10, outer=500),
+    "c3": dict(bs=1000, ts=16, outer=500),
+    "c4": dict(bs=100, ts=10, outer=500),
+}
+
+
+def parse():
+    p = argparse.ArgumentParser()
+    p.add_argument("--gpus", type=int, default=1)
+    p.add_argument("--steps", type=int, default=3)
+    p.add_argument("--warmup", type=int, default=1)
+    p.add_argument("--config", default="c2", choices=sorted(TUNED))
+    p.add_argument("--bs", type=int)
+    p.add_argument("--ts", type=int)
+    p.add_argument("--outer", type=int)
+    p.add_argument("--nq", type=int, help="use only the first NQ queries")
+    p.add_argument("--n", type=int, help="override the number of data points")
+    p.add_argument("--cpu-queries", type=int, default=512,
+                   help="queries in the CPU baseline sample")
+    p.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
+    p.add_argument("--build-reps", type=int, default=3)
+    return p.parse_args()
+
+
+def exact_knn_gpu(X, Q, k, chunk=1024):
+    """Exact k-NN by chunked fp32 matmul on the GPU (recall ground truth)."""
+    import torch
+    xn = (X * X).sum(1)
+    out = []
+    for s in range(0, Q.shape[0], chunk):
+        q = Q[s:s + chunk]
+        d2 = xn[None, :] - 2.0 * (q @ X.T)
+        out.append(d2.topk(k, dim=1, largest=False).indices)
+    return torch.cat(out)
+
+
+def recall_at_k(ids, gt):
+    hit = (ids[:, :, None] == gt[:, None, :]).any(2).float().sum().item()
+    return hit / gt.numel()
+
+
+def main():
+    a = parse()
+    if a.gpus != 1:
+        print("bench.py: this build runs on ONE GPU; --gpus %d is not supported "
+              "(every box in this pipeline has one GPU)" % a.gpus, file=sys.stderr)
+        sys.exit(2)
+    import numpy as np
+    import torch
+    if not torch.cuda.is_available():
+        print("bench.py needs a GPU", file=sys.stderr)
+        sys.exit(1)
+    import dciknn_cuda_amd as D
+    from dciknn_cuda_amd import _capi, workloads
+
+    cfg = dict(TUNED[a.config])
+    for key in ("bs", "ts", "outer"):
+        if getattr(a, key) is not None:
+            cfg[key] = getattr(a, key)
+    shape = dict(workloads.SHAPES[int(a.config[1])])
+    if a.n:
+        shape["n"] = a.n
+    gen = getattr(workloads, a.config)
+    X, Q = gen(n=shape["n"], nq=shape["nq"])
+    if a.nq:
+        Q = Q[:a.nq].contiguous()
+    N, dim = X.shape
+    nq = Q.shape[0]
+    M, L, k = shape["m"], shape["l"], shape["k"]
+    I = M * L
+    Xd, Qd = X.cuda(), Q.cuda()
+    torch.cuda.synchronize()
+
+    dci = D.DCI(dim, M, L, cfg["bs"], cfg["ts"], seed=4)
+    lib = dci._lib
+    _capi.check(lib.dcih_profile(dci._dci_inst, 1))
+    tms = (_capi.ctypes.c_float * _capi.NUM_TIMERS)()
+
+    # ---- build: projection + segmented sort --------------------------------
+    build_s, proj_ms, sort_ms = [], [], []
+    for rep in range(a.build_reps + 1):
+        dci.clear() if dci.num_points else None
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        dci.add(Xd)
+        torch.cuda.synchronize()
+        t1 = time.perf_counter()
+        _capi.check(lib.dcih_last_timings(dci._dci_inst, tms))
+        if rep:   # first one warms up allocator and code objects
+            build_s.append(t1 - t0)
+            proj_ms.append(tms[_capi.T_PROJECT])
+            sort_ms.append(tms[_capi.T_SEGSORT])
+    build_wall = float(np.median(build_s))
+    proj_t, sort_t = float(np.median(proj_ms)), float(np.median(sort_ms))
+
+    # ---- query: warmup, then K timed steps ----------------------------------
+    for _ in range(a.warmup):
+        dci.query(Qd, k, cfg["outer"])
+    trav_ms, merge_ms, qproj_ms = [], [], []
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(a.steps):
+        ids, dists = dci.query(Qd, k, cfg["outer"], return_int=True)
+        _capi.check(lib.dcih_last_timings(dci._dci_inst, tms))   # waits for this step's events
+        trav_ms.append(tms[_capi.T_TRAVERSE])
+        merge_ms.append(tms[_capi.T_MERGE])
+        qproj_ms.append(tms[_capi.T_QPROJECT])
+    torch.cuda.synchronize()
+    t1 = time.perf_counter()
+    ms_per_step = (t1 - t0) * 1e3 / a.steps
+    qps = nq / (ms_per_step * 1e-3)
+
+    # ---- outside the timed region: recall and traversal counters -------------
+    gt = exact_knn_gpu(Xd, Qd, k)
+    recall = recall_at_k(ids.long(), gt)
+    _, _, ctr = dci.query(Qd, k, cfg["outer"], return_int=True, return_counters=True)
+    torch.cuda.synchronize()
+    cm = ctr.double().mean(0).cpu().numpy()
+    V, C, S, steps_q = (float(v) for v in cm)
+
+    # algorithmic bytes of the traversal kernel per query: the query row, one
+    # key per search probe, one 4-byte id per visited entry, one data row per
+    # promoted point, k results.
+    bytes_per_query = 4 * dim + 4 * S + 4 * V + 4 * dim * C + 8 * k
+    trav_avg_ms = float(np.mean(trav_ms))
+    achieved = bytes_per_query * nq / (trav_avg_ms * 1e-3) / 1e9
+    roofline = dict(bound="hbm", kernel="traverse_kernel", achieved=achieved, peak=HBM_PEAK_GBS,
+                    unit="GB/s", frac=achieved / HBM_PEAK_GBS, traffic=None,
+                    bytes_per_launch=bytes_per_query * nq, avg_launch_ms=trav_avg_ms)
+    build_bytes_proj = 4.0 * N * (dim + I)
+    build_bytes_sort = 12.0 * N * I
+    build = dict(points_per_s=N / build_wall, wall_ms=build_wall * 1e3,
+                 project_ms=proj_t, segsort_ms=sort_t,
+                 project_gbs=build_bytes_proj / (proj_t * 1e-3) / 1e9,
+                 segsort_gbs=build_bytes_sort / (sort_t * 1e-3) / 1e9,
+                 project_frac=build_bytes_proj / (proj_t * 1e-3) / 1e9 / HBM_PEAK_GBS,
+                 segsort_frac=build_bytes_sort / (sort_t * 1e-3) / 1e9 / HBM_PEAK_GBS)
+
+    # ---- CPU baseline: the oracle on this box's host cores, bounded sample ----
+    cpu = None
+    if not a.no_cpu:
+        from oracle import dci_oracle as O
+        P = dci.directions.numpy()
+        Xn = X.numpy()
+        nqc = min(nq, a.cpu_queries)
+        Qn = Q[:nqc].numpy()
+        t0 = time.perf_counter()
+        skeys, sids = O.build_index(P, Xn, cfg["bs"])
+        t_build = time.perf_counter() - t0
+        qproj = O.project(Qn, P)
+        t0 = time.perf_counter()
+        ref = O.query(skeys, sids, Xn, Qn, qproj, M, L, cfg["bs"], cfg["ts"], k, cfg["outer"])
+        t_query = time.perf_counter() - t0
+        agree = float(np.mean([len(set(x.tolist()) & set(y.tolist())) / k
+                               for x, y in zip(ids[:nqc].cpu().numpy(), ref["ids"])]))
+        t0 = time.perf_counter()
+        Xt, Qt = torch.from_numpy(Xn), torch.from_numpy(Qn[:min(nqc, 128)])
+        torch.cdist(Qt, Xt).topk(k, largest=False)
+        t_exact = time.perf_counter() - t0
+        cpu = dict(value=nqc / t_query, unit="queries/s", cores=O.max_threads(), kind="port",
+                   sample="oracle (CPU restatement of the reference algorithm) on the first %d "
+                          "queries of the same workload, same (bs, ts, outer); build timed on "
+                          "all %d points" % (nqc, N),
+                   build_points_per_s=N / t_build, set_agreement_with_gpu=agree,
+                   exact_cdist_topk_queries_per_s=min(nqc, 128) / t_exact,
+                   host_cpus=os.cpu_count(), torch_threads=torch.get_num_threads())
+
+    out = {
+        "metric": "queries/sec at recall@10>=0.95, 1Mx128 fp32 k=10; index build points/sec"
+                  if a.config == "c2" else "queries/sec; index build points/sec",
+        "value": qps, "unit": "queries/s", "n_gpus": 1, "steps": a.steps, "warmup": a.warmup,
+        "ms_per_step": ms_per_step, "higher_is_better": True, "scaling": "weak",
+        "vs_baseline": None, "dtype": "f32", "data": "synthetic",
+        "config": {"workload": "%s: %d pts x %d fp32, %d queries, m=%d L=%d k=%d" %
+                               (a.config.upper(), N, dim, nq, M, L, k),
+                   "block_size": cfg["bs"], "thread_size": cfg["ts"],
+                   "num_outer_iterations": cfg["outer"]},
+        "recall_at_k": recall, "recall_ok": recall >= 0.95,
+        "build_points_per_s": N / build_wall,
+        "per_query": {"visited": V, "candidates": C, "probes": S, "outer_steps": steps_q,
+                      "algorithmic_bytes": bytes_per_query},
+        "kernel_ms": {"traverse": trav_avg_ms, "merge": float(np.mean(merge_ms)),
+                      "query_project": float(np.mean(qproj_ms))},
+        "build": build,
+        "roofline": roofline,
+        "cpu_baseline": cpu,
+    }
+    print(json.dumps(out))
+
+
+if __name__ == "__main__":
+    main()

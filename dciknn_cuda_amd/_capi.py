@@ -11,6 +11,8 @@ LIB_PATH = os.path.join(_HERE, "libdci_hip.so")
 
 NUM_COUNTERS = 4
 CTR_VISITED, CTR_CANDIDATES, CTR_PROBES, CTR_STEPS = range(4)
+NUM_TIMERS = 5
+T_PROJECT, T_SEGSORT, T_QPROJECT, T_TRAVERSE, T_MERGE = range(5)
 
 # name -> (restype, argtypes); one line per declaration in include/dci_hip.h
 _c = ctypes
@@ -27,6 +29,8 @@ SIGNATURES = {
                               _c.c_int, _c.c_int, _c.c_int, _c.c_int, _c.c_int,
                               _c.c_void_p, _c.c_void_p, _c.c_void_p, _c.c_void_p]),
     "dcih_get_index": (_c.c_int, [_c.c_void_p, _c.c_void_p, _c.c_void_p]),
+    "dcih_profile": (_c.c_int, [_c.c_void_p, _c.c_int]),
+    "dcih_last_timings": (_c.c_int, [_c.c_void_p, _c.c_void_p]),
     "dcih_num_points": (_c.c_int64, [_c.c_void_p]),
     "dcih_clear": (_c.c_int, [_c.c_void_p]),
     "dcih_reset": (_c.c_int, [_c.c_void_p]),

@@ -90,6 +90,10 @@ struct dcih_index {
     // grow-only query workspace
     void* ws = nullptr;
     size_t ws_bytes = 0;
+    // optional per-kernel timing: ev[2*t], ev[2*t+1] bracket timer t
+    bool profiling = false;
+    hipEvent_t ev[2 * DCIH_NUM_TIMERS] = {};
+    bool ev_valid[DCIH_NUM_TIMERS] = {};
 };
 
 namespace {
@@ -135,6 +139,13 @@ int ensure_ws(dcih_index* h, size_t bytes) {
 }
 
 size_t align_up(size_t v) { return (v + 255) & ~(size_t)255; }
+
+// Records the start (which = 0) or end (1) event of timer t when profiling.
+void mark(dcih_index* h, int t, int which, hipStream_t s) {
+    if (!h->profiling) return;
+    (void)hipEventRecord(h->ev[2 * t + which], s);
+    if (which) h->ev_valid[t] = true;
+}
 
 }  // namespace
 
@@ -212,9 +223,13 @@ int dcih_add(dcih_index* h, int dim, int64_t num_points, const float* d_data,
             rc = fail(DCIH_EHIP, "dcih_add: out of device memory");
             break;
         }
+        mark(h, DCIH_T_PROJECT, 0, s);
         rc = project(h->d_dirs, I, d_data, num_points, dim, d_keys, s);
+        mark(h, DCIH_T_PROJECT, 1, s);
         if (rc) break;
+        mark(h, DCIH_T_SEGSORT, 0, s);
         rc = segsort(d_keys, I, num_points, block_size, h->d_skeys, h->d_sids, d_tmp, s);
+        mark(h, DCIH_T_SEGSORT, 1, s);
     } while (0);
     // the scratch buffers are in use until the stream drains
     const hipError_t se = hipStreamSynchronize(s);
@@ -272,9 +287,45 @@ int dcih_query(dcih_index* h, int dim, int num_queries, const float* d_query,
     a.part = (unsigned long long*)(base + qp_bytes);
     a.gscratch = gs_bytes ? (uint32_t*)(base + qp_bytes + part_bytes) : nullptr;
 
+    mark(h, DCIH_T_QPROJECT, 0, s);
     rc = project(h->d_dirs, I, d_query, num_queries, dim, d_qproj, s);
+    mark(h, DCIH_T_QPROJECT, 1, s);
     if (rc) return rc;
-    return query(a, s);
+    hipEvent_t qev[3] = {h->ev[2 * DCIH_T_TRAVERSE], h->ev[2 * DCIH_T_TRAVERSE + 1],
+                         h->ev[2 * DCIH_T_MERGE + 1]};
+    rc = query(a, s, h->profiling ? qev : nullptr);
+    if (rc == DCIH_OK && h->profiling) {
+        // the merge starts where the traversal ends
+        h->ev_valid[DCIH_T_TRAVERSE] = h->ev_valid[DCIH_T_MERGE] = true;
+    }
+    return rc;
+}
+
+int dcih_profile(dcih_index* h, int enable) {
+    if (!h) return fail(DCIH_EINVAL, "dcih_profile: null handle");
+    DeviceGuard guard(h->device);
+    if (enable && !h->ev[0]) {
+        for (auto& e : h->ev) DCIH_HIP(hipEventCreate(&e));
+    }
+    h->profiling = enable != 0;
+    for (auto& v : h->ev_valid) v = false;
+    return DCIH_OK;
+}
+
+int dcih_last_timings(dcih_index* h, float* h_ms) {
+    if (!h || !h_ms) return fail(DCIH_EINVAL, "dcih_last_timings: null argument");
+    if (!h->profiling) return fail(DCIH_ESTATE, "dcih_last_timings: profiling is off");
+    DeviceGuard guard(h->device);
+    for (int t = 0; t < DCIH_NUM_TIMERS; t++) {
+        h_ms[t] = -1.0f;
+        if (!h->ev_valid[t]) continue;
+        // the merge timer shares its start with the traversal's end event
+        hipEvent_t a = t == DCIH_T_MERGE ? h->ev[2 * DCIH_T_TRAVERSE + 1] : h->ev[2 * t];
+        hipEvent_t b = h->ev[2 * t + 1];
+        DCIH_HIP(hipEventSynchronize(b));
+        DCIH_HIP(hipEventElapsedTime(&h_ms[t], a, b));
+    }
+    return DCIH_OK;
 }
 
 int dcih_get_index(const dcih_index* h, float* h_keys, int32_t* h_ids) {
@@ -311,6 +362,7 @@ int dcih_free(dcih_index* h) {
     (void)release_index(h);
     if (h->ws) (void)hipFree(h->ws);
     if (h->d_dirs) (void)hipFree(h->d_dirs);
+    for (auto& e : h->ev) if (e) (void)hipEventDestroy(e);
     delete h;
     return DCIH_OK;
 }

@@ -38,6 +38,8 @@ struct QueryArgs {
 size_t query_part_bytes(const QueryArgs& a);
 // Bytes of global counter scratch the traversal needs (0 when LDS suffices).
 size_t query_gscratch_bytes(const QueryArgs& a);
-int query(const QueryArgs& a, hipStream_t s);
+// ev: null, or three events recorded before the traversal, between traversal
+// and merge, and after the merge.
+int query(const QueryArgs& a, hipStream_t s, hipEvent_t* ev);
 
 }  // namespace dcih

@@ -325,7 +325,7 @@ size_t query_gscratch_bytes(const QueryArgs& a) {
     return (size_t)traverse_grid(a, y) * (size_t)y.counter_words * 4;
 }
 
-int query(const QueryArgs& a, hipStream_t s) {
+int query(const QueryArgs& a, hipStream_t s, hipEvent_t* ev) {
     if (a.nq <= 0) return 0;
     if (a.k > 8192) return fail(-4, "query: num_neighbours above 8192 is not supported");
     if ((int64_t)a.M * a.ppb * 8 > 0x7fffffffLL)
@@ -349,6 +349,7 @@ int query(const QueryArgs& a, hipStream_t s) {
                            dim3(256), 0, s, a.counters, cells);
     }
     const int64_t grid = traverse_grid(a, y);
+    if (ev) (void)hipEventRecord(ev[0], s);
     if (y.lds_counters) {
         hipLaunchKernelGGL(traverse_kernel<true>, dim3((unsigned)grid), dim3(kWave), y.lds_bytes, s, a, y);
     } else {
@@ -356,9 +357,11 @@ int query(const QueryArgs& a, hipStream_t s) {
         hipLaunchKernelGGL(traverse_kernel<false>, dim3((unsigned)grid), dim3(kWave), y.lds_bytes, s, a, y);
     }
     DCIH_HIP(hipGetLastError());
+    if (ev) (void)hipEventRecord(ev[1], s);
     const int cap = merge_cap(a.k);
     hipLaunchKernelGGL(merge_topk_kernel, dim3((unsigned)a.nq), dim3(kMergeThreads),
                        (size_t)cap * sizeof(unsigned long long), s, a, cap);
+    if (ev) (void)hipEventRecord(ev[2], s);
     DCIH_HIP(hipGetLastError());
     return 0;
 }

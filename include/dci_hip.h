@@ -39,6 +39,16 @@ enum {
     DCIH_NUM_COUNTERS = 4
 };
 
+/* Kernels timed by dcih_profile / dcih_last_timings. */
+enum {
+    DCIH_T_PROJECT = 0,   /* build: projection of the data            */
+    DCIH_T_SEGSORT = 1,   /* build: segmented sort                    */
+    DCIH_T_QPROJECT = 2,  /* query: projection of the queries         */
+    DCIH_T_TRAVERSE = 3,  /* query: traversal + distances + top-k     */
+    DCIH_T_MERGE = 4,     /* query: merge of the per-partition top-k  */
+    DCIH_NUM_TIMERS = 5
+};
+
 /* Message for the last failing call on this thread ("" if none). */
 const char* dcih_last_error(void);
 
@@ -101,6 +111,16 @@ int dcih_query(dcih_index* h, int dim, int num_queries, const float* d_query,
  * either pointer may be NULL.  Synchronous.
  */
 int dcih_get_index(const dcih_index* h, float* h_keys, int32_t* h_ids);
+
+/*
+ * Per-kernel timing with HIP events on the caller's stream (no counterpart in
+ * the reference).  After dcih_profile(h, 1) every dcih_add / dcih_query
+ * brackets its kernels with events; dcih_last_timings waits for them and
+ * writes DCIH_NUM_TIMERS durations in milliseconds (-1 for a kernel that has
+ * not run since profiling was switched on).
+ */
+int dcih_profile(dcih_index* h, int enable);
+int dcih_last_timings(dcih_index* h, float* h_ms);
 
 /* Number of points currently indexed (0 when empty). */
 int64_t dcih_num_points(const dcih_index* h);
