@@ -1,0 +1,151 @@
+"""GPU tests of the Python surface kept from dciknn_cuda/core.py:25-169."""
+import numpy as np
+import pytest
+import torch
+
+pytestmark = pytest.mark.gpu
+
+
+def _xy(n=2000, nq=20, dim=16, seed=0):
+    g = torch.Generator().manual_seed(seed)
+    x = torch.randn(n + nq, dim, generator=g)
+    return x[:n].cuda(), x[n:].cuda()
+
+
+def test_query_return_contract(gpu):
+    X, Q = _xy()
+    dci = gpu.DCI(16, 2, 5, 10, 8)
+    assert (dci.dim, dci.num_comp_indices, dci.num_simp_indices) == (16, 2, 5)
+    dci.add(X)
+    assert dci.num_points == 2000
+    idx, dist = dci.query(Q, 7, 50)
+    assert idx.shape == (20, 7) and dist.shape == (20, 7)
+    assert idx.dtype == torch.float32 and dist.dtype == torch.float32   # ids come back as floats
+    assert idx.is_cuda and dist.is_cuda
+    assert torch.all(dist[:, 1:] >= dist[:, :-1])
+    # returned distance belongs to the returned id
+    d = (X[idx.long()] - Q[:, None, :]).norm(dim=2)
+    assert torch.allclose(d, dist, rtol=1e-5, atol=1e-6)
+    # 1-D query is treated as one row
+    i1, d1 = dci.query(Q[3], 7, 50)
+    assert i1.shape == (1, 7) and torch.equal(i1[0], idx[3]) and torch.equal(d1[0], dist[3])
+    dci.free()
+
+
+def test_second_add_raises_and_clear_allows_again(gpu):
+    X, Q = _xy()
+    dci = gpu.DCI(16, 2, 5, 10, 8)
+    dci.add(X)
+    with pytest.raises(RuntimeError):
+        dci.add(X)
+    a = dci.query(Q, 3, 20)
+    dci.clear()
+    assert dci.num_points == 0
+    with pytest.raises(RuntimeError):
+        dci.query(Q, 3, 20)
+    dci.add(X)
+    b = dci.query(Q, 3, 20)
+    assert torch.equal(a[0], b[0]) and torch.equal(a[1], b[1])   # same directions after clear()
+
+
+def test_reset_draws_new_seeded_directions(gpu):
+    d1 = gpu.DCI(16, 2, 5, 10, 8, seed=5)
+    d2 = gpu.DCI(16, 2, 5, 10, 8, seed=5)
+    d3 = gpu.DCI(16, 2, 5, 10, 8, seed=6)
+    p1 = d1.directions
+    assert torch.equal(p1, d2.directions) and not torch.equal(p1, d3.directions)
+    assert torch.allclose(p1.double().norm(dim=1), torch.ones(10, dtype=torch.float64), atol=2e-6)
+    d1.reset(); d2.reset()
+    assert not torch.equal(d1.directions, p1)
+    assert torch.equal(d1.directions, d2.directions)    # the sequence itself is seeded
+
+
+def test_directions_look_isotropic(gpu):
+    """Entries of unit Gaussian directions in dim d have mean 0 and variance 1/d."""
+    p = gpu.DCI(256, 8, 16, seed=1).directions.double()
+    assert abs(p.mean().item()) < 3.0 / np.sqrt(p.numel() * 256)
+    assert abs(p.var().item() * 256 - 1.0) < 0.02
+    gram = p @ p.T - torch.eye(128, dtype=torch.float64)
+    assert gram.abs().max().item() < 0.4                # no two directions nearly parallel
+
+
+def test_set_directions_round_trip_and_shape_check(gpu):
+    dci = gpu.DCI(4, 1, 2, 1, 1)
+    dci.directions = torch.tensor([[1., 0, 0, 0], [0, 1., 0, 0]])
+    assert torch.equal(dci.directions, torch.tensor([[1., 0, 0, 0], [0, 1., 0, 0]]))
+    with pytest.raises(ValueError):
+        dci.directions = torch.zeros(3, 4)
+    X = torch.tensor([[0., 0, 0, 0], [1, 3, 0, 0], [2, 1, 0, 0], [5, 5, 0, 0]]).cuda()
+    dci.add(X)
+    with pytest.raises(RuntimeError):
+        dci.directions = torch.zeros(2, 4)              # not while points are indexed
+    # the hand-derived traversal of tests/golden (k=2): ids [2, 0]
+    idx, dist = dci.query(torch.tensor([[1.4, 1.2, 0, 0]]).cuda(), 2, 1, return_int=True)
+    assert idx.tolist() == [[2, 0]]
+    np.testing.assert_allclose(dist.cpu().numpy(), [[0.6324555, 1.8439089]], rtol=1e-6)
+
+
+def test_argument_errors(gpu):
+    X, Q = _xy()
+    dci = gpu.DCI(16, 2, 5, 10, 8)
+    with pytest.raises(ValueError):
+        dci.add(X[:, :8].contiguous())
+    with pytest.raises(TypeError):
+        dci.add(X.double())
+    with pytest.raises(TypeError):
+        dci.add(X.cpu())
+    with pytest.raises(ValueError):
+        dci.add(X.t().contiguous().t())
+    dci.add(X)
+    with pytest.raises(TypeError):
+        dci.query(Q, 2.5)
+    with pytest.raises(ValueError):
+        dci.query(Q, 0)
+    with pytest.raises(ValueError):
+        dci.query(Q, 2001)
+    with pytest.raises(NotImplementedError):
+        dci.query(Q, 3, blind=True)
+    dci._block_size = 11                                # partitioning is part of the index
+    from dciknn_cuda_amd._capi import DCIError
+    with pytest.raises(DCIError):
+        dci.query(Q, 3)
+
+
+def test_all_neighbours_default(gpu):
+    """num_neighbours=-1 means every indexed point, ranked (core.py:84-85)."""
+    X, Q = _xy(n=300, nq=4)
+    dci = gpu.DCI(16, 2, 3, 4, 4)
+    dci.add(X)
+    idx, dist = dci.query(Q, num_outer_iterations=10 ** 6)
+    assert idx.shape == (4, 300)
+    want = torch.cdist(Q, X).sort(dim=1)
+    assert torch.allclose(dist, want.values, rtol=1e-5, atol=1e-6)
+    assert torch.equal(idx.long().sort(dim=1).values, torch.arange(300).cuda().expand(4, 300))
+
+
+def test_mdci_single_device_equals_dci(gpu):
+    X, Q = _xy()
+    m = gpu.MDCI(16, 2, 5, 10, 8, devices=[0])
+    d = gpu.DCI(16, 2, 5, 10, 8, device=0)
+    m.add(X.cpu())          # MDCI moves the shard itself (core.py:125)
+    d.add(X)
+    mi, md = m.query(Q.cpu(), 5, 30)
+    di, dd = d.query(Q, 5, 30)
+    assert torch.equal(mi, di) and torch.equal(md, dd)
+    with pytest.raises(RuntimeError):
+        m.query(Q, -1)
+    m.clear(); m.reset(); m.free()
+
+
+def test_non_default_stream(gpu, oracle):
+    """Work is enqueued on torch's current stream."""
+    X, Q = _xy()
+    dci = gpu.DCI(16, 2, 5, 10, 8)
+    s = torch.cuda.Stream()
+    torch.cuda.synchronize()
+    with torch.cuda.stream(s):
+        dci.add(X)
+        i1, d1 = dci.query(Q, 5, 30)
+    s.synchronize()
+    i0, d0 = dci.query(Q, 5, 30)
+    assert torch.equal(i0, i1) and torch.equal(d0, d1)

@@ -1,0 +1,129 @@
+"""Host-side checks that need no GPU: the C-ABI library loads and exports what
+include/dci_hip.h declares, argument errors come back as status codes, and the
+Python front end validates its inputs like dciknn_cuda/core.py:53-92 does."""
+import ctypes
+import os
+import re
+
+import pytest
+import torch
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+
+
+def _declared():
+    text = open(os.path.join(ROOT, "include", "dci_hip.h")).read()
+    text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
+    return sorted(set(re.findall(r"\b(dcih_[a-z_]+)\s*\(", text)))
+
+
+def test_library_exports_every_declared_symbol():
+    from dciknn_cuda_amd import _capi
+    lib = ctypes.CDLL(_capi.LIB_PATH)
+    names = _declared()
+    assert len(names) >= 15
+    for name in names:
+        assert hasattr(lib, name), "libdci_hip.so lacks %s" % name
+        assert name in _capi.SIGNATURES, "no ctypes signature for %s" % name
+    assert set(_capi.SIGNATURES) == set(names)
+    assert _capi.lib().dcih_abi_version() == 1
+
+
+def test_null_and_bad_arguments_return_status_codes():
+    """No compute: only paths that fail before any HIP call."""
+    from dciknn_cuda_amd import _capi
+    lib = _capi.lib()
+    assert lib.dcih_add(None, 4, 10, None, 1, 1, None) == -1
+    assert b"null handle" in lib.dcih_last_error()
+    assert lib.dcih_query(None, 4, 1, None, 1, 0, 1, 10, 1, 1, None, None, None, None) == -1
+    assert lib.dcih_create(0, 1, 1, 0, 0, ctypes.byref(ctypes.c_void_p())) == -1
+    assert lib.dcih_create(4, 1, 1, 0, 0, None) == -1
+    assert lib.dcih_project(None, 1, None, 1, 1, None, None) == -1
+    assert lib.dcih_segsort(None, 1, 1, 1, None, None, None) == -1
+    assert lib.dcih_free(None) == 0
+    assert lib.dcih_num_points(None) == 0
+    with pytest.raises(_capi.DCIError):
+        _capi.check(lib.dcih_clear(None))
+
+
+def test_constructor_needs_a_gpu():
+    if torch.cuda.is_available():
+        pytest.skip("a GPU is present")
+    from dciknn_cuda_amd import DCI
+    with pytest.raises(RuntimeError):
+        DCI(8)
+
+
+def _bare(dim=4):
+    """A DCI object without a device handle, for the pure-Python validation."""
+    from dciknn_cuda_amd import DCI
+    d = DCI.__new__(DCI)
+    d._dim, d._num_comp_indices, d._num_simp_indices = dim, 2, 3
+    d._dci_inst, d._array, d.num_points = None, None, 0
+    return d
+
+
+def test_check_data_exception_types():
+    d = _bare(4)
+
+    class FakeCuda(torch.Tensor):
+        @property
+        def is_cuda(self):
+            return True
+
+    ok = torch.zeros(3, 4).as_subclass(FakeCuda)
+    d._check_data(ok)
+    with pytest.raises(ValueError):
+        d._check_data(torch.zeros(3, 5).as_subclass(FakeCuda))            # wrong dim
+    with pytest.raises(TypeError):
+        d._check_data(torch.zeros(3, 4, dtype=torch.float64).as_subclass(FakeCuda))
+    with pytest.raises(ValueError):
+        d._check_data(torch.zeros(4, 3).t().as_subclass(FakeCuda))         # not C-contiguous
+    with pytest.raises(TypeError):
+        d._check_data(torch.zeros(3, 4))                                   # not on the GPU
+
+
+def test_positive_integer_rule():
+    d = _bare()
+    d._ensure_positive_integer(3)
+    with pytest.raises(TypeError):
+        d._ensure_positive_integer(3.0)
+    with pytest.raises(ValueError):
+        d._ensure_positive_integer(0)
+
+
+def test_freed_instance_raises():
+    d = _bare()
+    with pytest.raises(RuntimeError):
+        d.add(torch.zeros(2, 4))
+    with pytest.raises(RuntimeError):
+        d.query(torch.zeros(2, 4), 1)
+
+
+def test_mdci_accepts_one_device_only():
+    from dciknn_cuda_amd import MDCI
+    with pytest.raises(NotImplementedError):
+        MDCI(8, devices=[0, 1])
+    with pytest.raises(NotImplementedError):
+        MDCI(8, devices=[])
+
+
+def test_import_name_of_the_reference_package():
+    import dciknn_cuda
+    import dciknn_cuda_amd
+    assert dciknn_cuda.DCI is dciknn_cuda_amd.DCI and dciknn_cuda.MDCI is dciknn_cuda_amd.MDCI
+
+
+def test_workload_generators_are_seeded():
+    from dciknn_cuda_amd import workloads
+    a, qa = workloads.c2(n=2000, nq=10)
+    b, qb = workloads.c2(n=2000, nq=10)
+    assert torch.equal(a, b) and torch.equal(qa, qb)
+    assert a.shape == (2000, 128) and a.min() >= 0 and torch.equal(a, a.round())
+    x, q = workloads.c1(n=300, nq=20)
+    assert x.shape == (300, 100) and q.shape == (20, 100)
+    x3, _ = workloads.c3(n=1000, nq=10)
+    assert torch.allclose(x3.norm(dim=1), torch.ones(1000), atol=1e-5)
+    x4, _ = workloads.c4(n=500, nq=5)
+    assert x4.shape == (500, 960)
+    assert workloads.c5_batch(0, n=100).shape == (100, 64)
