@@ -11,6 +11,8 @@ LIB_PATH = os.path.join(_HERE, "libdci_hip.so")
 
 NUM_COUNTERS = 4
 CTR_VISITED, CTR_CANDIDATES, CTR_PROBES, CTR_STEPS = range(4)
+OPT_TRAVERSAL = 0
+TRAVERSAL_AUTO, TRAVERSAL_STEP, TRAVERSAL_BATCH = 0, 1, 2
 NUM_TIMERS = 5
 T_PROJECT, T_SEGSORT, T_QPROJECT, T_TRAVERSE, T_MERGE = range(5)
 
@@ -29,6 +31,8 @@ SIGNATURES = {
                               _c.c_int, _c.c_int, _c.c_int, _c.c_int, _c.c_int,
                               _c.c_void_p, _c.c_void_p, _c.c_void_p, _c.c_void_p]),
     "dcih_get_index": (_c.c_int, [_c.c_void_p, _c.c_void_p, _c.c_void_p]),
+    "dcih_set_option": (_c.c_int, [_c.c_void_p, _c.c_int, _c.c_int]),
+    "dcih_phase_profile": (_c.c_int, [_c.c_void_p, _c.c_void_p]),
     "dcih_profile": (_c.c_int, [_c.c_void_p, _c.c_int]),
     "dcih_last_timings": (_c.c_int, [_c.c_void_p, _c.c_void_p]),
     "dcih_num_points": (_c.c_int64, [_c.c_void_p]),

@@ -5,7 +5,8 @@ dciknn_cuda/core.py:25-169 (argument names, defaults, exception types, return
 shapes and dtypes) on top of libdci_hip.so.  Additions, all keyword-only and
 optional: `seed` / `directions` at construction and the `directions` property
 (the reference can neither seed, inject nor read its directions), and
-`return_int` / `return_counters` on `query`.
+`return_int` / `return_counters` on `query`, and `traversal` / `set_traversal`
+to pick the query kernel.
 """
 import torch
 
@@ -19,7 +20,7 @@ def _stream_ptr(device):
 class DCI(object):
 
     def __init__(self, dim, num_comp_indices=2, num_simp_indices=7, bs=100, ts=10, device=0,
-                 *, seed=0, directions=None):
+                 *, seed=0, directions=None, traversal="auto"):
         if not torch.cuda.is_available():
             raise RuntimeError("DCI requires GPU access, please check the ROCm driver.")
         self._dim = dim
@@ -39,6 +40,8 @@ class DCI(object):
         self.num_points = 0
         if directions is not None:
             self.directions = directions
+        if traversal != "auto":
+            self.set_traversal(traversal)
 
     def __del__(self):
         try:
@@ -75,6 +78,15 @@ class DCI(object):
         if tuple(value.shape) != want:
             raise ValueError("directions must have shape %s" % (want,))
         _capi.check(self._lib.dcih_set_directions(self._dci_inst, value.data_ptr()))
+
+    def set_traversal(self, mode):
+        """Pick the query kernel: "auto", "step" (one wavefront per partition,
+        one window per step) or "batch" (one workgroup per partition, whole index
+        ranges per epoch).  Both return the same neighbours."""
+        self._require_handle()
+        value = {"auto": _capi.TRAVERSAL_AUTO, "step": _capi.TRAVERSAL_STEP,
+                 "batch": _capi.TRAVERSAL_BATCH}[mode]
+        _capi.check(self._lib.dcih_set_option(self._dci_inst, _capi.OPT_TRAVERSAL, value))
 
     def _require_handle(self):
         if self._dci_inst is None:

@@ -87,6 +87,10 @@ struct dcih_index {
     int block_size = 0;
     float* d_skeys = nullptr;           // [I][n]
     int32_t* d_sids = nullptr;          // [I][n]
+    uint32_t* d_inv = nullptr;          // [I][n] position of each point in its sorted slice
+    uint16_t* d_lids = nullptr;         // [I][n] partition-relative ids (partitions <= 65536 points)
+    int traversal = 0;                  // DCIH_OPT_TRAVERSAL value
+    unsigned long long* d_phase_ticks = nullptr;   // optional profile of the batch kernel
     // grow-only query workspace
     void* ws = nullptr;
     size_t ws_bytes = 0;
@@ -124,6 +128,8 @@ int draw_directions(dcih_index* h) {
 int release_index(dcih_index* h) {
     if (h->d_skeys) { DCIH_HIP(hipFree(h->d_skeys)); h->d_skeys = nullptr; }
     if (h->d_sids) { DCIH_HIP(hipFree(h->d_sids)); h->d_sids = nullptr; }
+    if (h->d_inv) { DCIH_HIP(hipFree(h->d_inv)); h->d_inv = nullptr; }
+    if (h->d_lids) { DCIH_HIP(hipFree(h->d_lids)); h->d_lids = nullptr; }
     h->d_data = nullptr;
     h->n = 0;
     h->block_size = 0;
@@ -214,10 +220,14 @@ int dcih_add(dcih_index* h, int dim, int64_t num_points, const float* d_data,
     float* d_keys = nullptr;
     void* d_tmp = nullptr;
     const size_t tmp_bytes = segsort_tmp_bytes(I, num_points, block_size);
+    const bool small_parts = (num_points + block_size - 1) / block_size <= 65536;
     int rc = DCIH_OK;
     do {
         if (hipMalloc(&h->d_skeys, cells * sizeof(float)) != hipSuccess ||
             hipMalloc(&h->d_sids, cells * sizeof(int32_t)) != hipSuccess ||
+            hipMalloc(&h->d_inv, cells * sizeof(uint32_t)) != hipSuccess ||
+            // +16: the traversal reads whole aligned 16-byte chunks, also at the very end
+            (small_parts && hipMalloc(&h->d_lids, (cells + 16) * sizeof(uint16_t)) != hipSuccess) ||
             hipMalloc(&d_keys, cells * sizeof(float)) != hipSuccess ||
             (tmp_bytes && hipMalloc(&d_tmp, tmp_bytes) != hipSuccess)) {
             rc = fail(DCIH_EHIP, "dcih_add: out of device memory");
@@ -228,7 +238,7 @@ int dcih_add(dcih_index* h, int dim, int64_t num_points, const float* d_data,
         mark(h, DCIH_T_PROJECT, 1, s);
         if (rc) break;
         mark(h, DCIH_T_SEGSORT, 0, s);
-        rc = segsort(d_keys, I, num_points, block_size, h->d_skeys, h->d_sids, d_tmp, s);
+        rc = segsort(d_keys, I, num_points, block_size, h->d_skeys, h->d_sids, h->d_inv, h->d_lids, d_tmp, s);
         mark(h, DCIH_T_SEGSORT, 1, s);
     } while (0);
     // the scratch buffers are in use until the stream drains
@@ -265,7 +275,9 @@ int dcih_query(dcih_index* h, int dim, int num_queries, const float* d_query,
     const int I = num_indices(h);
 
     QueryArgs a;
-    a.skeys = h->d_skeys; a.sids = h->d_sids; a.data = h->d_data; a.query = d_query;
+    a.skeys = h->d_skeys; a.sids = h->d_sids; a.inv = h->d_inv; a.lids = h->d_lids; a.data = h->d_data; a.query = d_query;
+    a.mode = h->traversal; a.item_list = nullptr; a.item_count = nullptr;
+    a.phase_ticks = h->d_phase_ticks;
     a.N = h->n;
     a.ppb = (h->n + block_size - 1) / block_size;
     a.dim = dim; a.M = h->M; a.L = h->L; a.B = block_size; a.T = thread_size;
@@ -279,13 +291,16 @@ int dcih_query(dcih_index* h, int dim, int num_queries, const float* d_query,
     const size_t qp_bytes = align_up((size_t)I * num_queries * sizeof(float));
     const size_t part_bytes = align_up(query_part_bytes(a));
     const size_t gs_bytes = align_up(query_gscratch_bytes(a));
-    int rc = ensure_ws(h, qp_bytes + part_bytes + gs_bytes);
+    const size_t redo_bytes = align_up((size_t)num_queries * block_size * sizeof(int32_t));
+    int rc = ensure_ws(h, qp_bytes + part_bytes + gs_bytes + redo_bytes + 256);
     if (rc) return rc;
     char* base = (char*)h->ws;
     float* d_qproj = (float*)base;
     a.qproj = d_qproj;
     a.part = (unsigned long long*)(base + qp_bytes);
     a.gscratch = gs_bytes ? (uint32_t*)(base + qp_bytes + part_bytes) : nullptr;
+    a.redo_items = (int32_t*)(base + qp_bytes + part_bytes + gs_bytes);
+    a.redo_count = (uint32_t*)(base + qp_bytes + part_bytes + gs_bytes + redo_bytes);
 
     mark(h, DCIH_T_QPROJECT, 0, s);
     rc = project(h->d_dirs, I, d_query, num_queries, dim, d_qproj, s);
@@ -299,6 +314,21 @@ int dcih_query(dcih_index* h, int dim, int num_queries, const float* d_query,
         h->ev_valid[DCIH_T_TRAVERSE] = h->ev_valid[DCIH_T_MERGE] = true;
     }
     return rc;
+}
+
+int dcih_set_option(dcih_index* h, int option, int value) {
+    if (!h) return fail(DCIH_EINVAL, "dcih_set_option: null handle");
+    if (option == DCIH_OPT_TRAVERSAL && value >= 0 && value <= 2) {
+        h->traversal = value;
+        return DCIH_OK;
+    }
+    return fail(DCIH_EINVAL, "dcih_set_option: unknown option or value");
+}
+
+int dcih_phase_profile(dcih_index* h, uint64_t* d_ticks) {
+    if (!h) return fail(DCIH_EINVAL, "dcih_phase_profile: null handle");
+    h->d_phase_ticks = (unsigned long long*)d_ticks;
+    return DCIH_OK;
 }
 
 int dcih_profile(dcih_index* h, int enable) {
@@ -382,7 +412,7 @@ int dcih_segsort(const float* d_keys, int num_idx, int64_t num_points, int block
     const size_t tmp_bytes = segsort_tmp_bytes(num_idx, num_points, block_size);
     void* d_tmp = nullptr;
     if (tmp_bytes) DCIH_HIP(hipMalloc(&d_tmp, tmp_bytes));
-    const int rc = segsort(d_keys, num_idx, num_points, block_size, d_skeys, d_sids, d_tmp, s);
+    const int rc = segsort(d_keys, num_idx, num_points, block_size, d_skeys, d_sids, nullptr, nullptr, d_tmp, s);
     if (d_tmp) {
         (void)hipStreamSynchronize(s);
         (void)hipFree(d_tmp);

@@ -14,12 +14,19 @@ int project(const float* d_dirs, int num_dirs, const float* d_rows, int64_t num_
 // (key, id).  d_tmp is scratch of segsort_tmp_bytes() bytes (may be null when
 // that is 0).
 size_t segsort_tmp_bytes(int num_indices, int64_t n, int block_size);
+// d_inv: null, or [num_indices][n] receiving each point's position inside its
+// sorted slice (the inverse of d_sids).  d_lids: null, or [num_indices][n]
+// receiving the ids relative to their partition's first point as 16-bit values
+// (only meaningful when a partition holds at most 65536 points).
 int segsort(const float* d_keys, int num_indices, int64_t n, int block_size,
-            float* d_skeys, int32_t* d_sids, void* d_tmp, hipStream_t s);
+            float* d_skeys, int32_t* d_sids, uint32_t* d_inv, uint16_t* d_lids, void* d_tmp,
+            hipStream_t s);
 
 struct QueryArgs {
     const float* skeys;      // [I][N] sorted projections
     const int32_t* sids;     // [I][N] point ids in the same order
+    const uint32_t* inv;     // [I][N] position of every point inside its sorted slice
+    const uint16_t* lids;    // [I][N] ids relative to the partition start (null if ppb > 65536)
     const float* data;       // [N][dim]
     const float* query;      // [nq][dim]
     const float* qproj;      // [I][nq]
@@ -32,12 +39,23 @@ struct QueryArgs {
     unsigned long long* part;      // [nq][B][kcap] packed (dist bits << 32 | id)
     unsigned long long* counters;  // null or [nq][4]
     uint32_t* gscratch;      // global visit counters when they do not fit LDS
+    int32_t* redo_items;     // [nq*B] (query, partition) pairs the batch kernel hands back
+    uint32_t* redo_count;    // their number
+    const int32_t* item_list;    // step-by-step kernel: null = all nq*B items, else this list
+    const uint32_t* item_count;  // ... of this length
+    unsigned long long* phase_ticks;  // null, or 16 accumulators for the batch kernel's phases
+    int mode;                // 0 = pick, 1 = step-by-step kernel, 2 = batch kernel
     int32_t* out_ids;        // [nq][k]
     float* out_dists;        // [nq][k]
 };
 size_t query_part_bytes(const QueryArgs& a);
 // Bytes of global counter scratch the traversal needs (0 when LDS suffices).
 size_t query_gscratch_bytes(const QueryArgs& a);
+// Batch traversal (traverse_block.hip): whether the shape fits its fixed LDS
+// tables, and the launch itself.
+bool block_traversal_supported(const QueryArgs& a, size_t* lds_bytes);
+int query_block(const QueryArgs& a, hipStream_t s);
+
 // ev: null, or three events recorded before the traversal, between traversal
 // and merge, and after the merge.
 int query(const QueryArgs& a, hipStream_t s, hipEvent_t* ev);

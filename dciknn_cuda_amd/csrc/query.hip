@@ -107,11 +107,12 @@ __global__ __launch_bounds__(kWave) void traverse_kernel(QueryArgs a, Layout y) 
         reinterpret_cast<unsigned long long*>(smem + ((y.state_bytes + 15) & ~15));
     uint32_t* s_cnt = reinterpret_cast<uint32_t*>(smem + ((y.state_bytes + 15) & ~15) + y.topk_bytes);
 
-    const int64_t items = (int64_t)a.nq * a.B;
+    const int64_t items = a.item_list ? (int64_t)*a.item_count : (int64_t)a.nq * a.B;
     const uint32_t cmask = y.cbits == 32 ? 0xffffffffu : ((1u << y.cbits) - 1u);
     const int fshift = y.cbits == 4 ? 3 : (y.cbits == 8 ? 2 : (y.cbits == 16 ? 1 : 0));  // log2(fields/word)
 
-    for (int64_t item = blockIdx.x; item < items; item += gridDim.x) {
+    for (int64_t slot = blockIdx.x; slot < items; slot += gridDim.x) {
+        const int64_t item = a.item_list ? (int64_t)a.item_list[slot] : slot;
         const int b = (int)(item % a.B);
         const int qi = (int)(item / a.B);
         const int64_t off = (int64_t)b * a.ppb;
@@ -296,9 +297,10 @@ __global__ __launch_bounds__(kMergeThreads) void merge_topk_kernel(QueryArgs a, 
     }
 }
 
-__global__ void zero_u64_kernel(unsigned long long* p, int64_t n) {
+__global__ void zero_u64_kernel(unsigned long long* p, int64_t n, uint32_t* also) {
     const int64_t stride = (int64_t)gridDim.x * blockDim.x;
     for (int64_t e = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; e < n; e += stride) p[e] = 0;
+    if (also && blockIdx.x == 0 && threadIdx.x == 0) *also = 0;
 }
 
 int merge_cap(int k) {
@@ -325,7 +327,8 @@ size_t query_gscratch_bytes(const QueryArgs& a) {
     return (size_t)traverse_grid(a, y) * (size_t)y.counter_words * 4;
 }
 
-int query(const QueryArgs& a, hipStream_t s, hipEvent_t* ev) {
+int query(const QueryArgs& a_in, hipStream_t s, hipEvent_t* ev) {
+    QueryArgs a = a_in;
     if (a.nq <= 0) return 0;
     if (a.k > 8192) return fail(-4, "query: num_neighbours above 8192 is not supported");
     if ((int64_t)a.M * a.ppb * 8 > 0x7fffffffLL)
@@ -333,6 +336,10 @@ int query(const QueryArgs& a, hipStream_t s, hipEvent_t* ev) {
     const Layout y = make_layout(a);
     if (y.lds_bytes > (size_t)kMaxLds)
         return fail(-4, "query: dim / num_indices / num_neighbours too large for LDS state");
+    const bool can_block = block_traversal_supported(a, nullptr);
+    if (a.mode == 2 && !can_block)
+        return fail(-4, "query: this shape does not fit the batch traversal kernel");
+    const bool use_block = a.mode != 1 && can_block;
     static bool attr_done = false;
     if (!attr_done) {
         DCIH_HIP(hipFuncSetAttribute((const void*)traverse_kernel<true>,
@@ -343,18 +350,30 @@ int query(const QueryArgs& a, hipStream_t s, hipEvent_t* ev) {
                                      hipFuncAttributeMaxDynamicSharedMemorySize, kMaxLds));
         attr_done = true;
     }
-    if (a.counters) {
-        const int64_t cells = (int64_t)a.nq * 4;
-        hipLaunchKernelGGL(zero_u64_kernel, dim3((unsigned)min((int64_t)1024, (cells + 255) / 256)),
-                           dim3(256), 0, s, a.counters, cells);
+    {   // zero the counters and the redo count with a kernel (safe under graph capture)
+        const int64_t cells = a.counters ? (int64_t)a.nq * 4 : 0;
+        hipLaunchKernelGGL(zero_u64_kernel, dim3((unsigned)max((int64_t)1, min((int64_t)1024, (cells + 255) / 256))),
+                           dim3(256), 0, s, a.counters, cells, a.redo_count);
     }
-    const int64_t grid = traverse_grid(a, y);
     if (ev) (void)hipEventRecord(ev[0], s);
-    if (y.lds_counters) {
+    a.item_list = nullptr;
+    a.item_count = nullptr;
+    if (use_block) {
+        const int rc = query_block(a, s);
+        if (rc) return rc;
+        // whatever the batch kernel handed back goes through the step-by-step kernel
+        a.item_list = a.redo_items;
+        a.item_count = a.redo_count;
+        const int64_t grid = min((int64_t)a.nq * a.B, (int64_t)1024);
         hipLaunchKernelGGL(traverse_kernel<true>, dim3((unsigned)grid), dim3(kWave), y.lds_bytes, s, a, y);
     } else {
-        if (!a.gscratch) return fail(-1, "query: counter scratch missing");
-        hipLaunchKernelGGL(traverse_kernel<false>, dim3((unsigned)grid), dim3(kWave), y.lds_bytes, s, a, y);
+        const int64_t grid = traverse_grid(a, y);
+        if (y.lds_counters) {
+            hipLaunchKernelGGL(traverse_kernel<true>, dim3((unsigned)grid), dim3(kWave), y.lds_bytes, s, a, y);
+        } else {
+            if (!a.gscratch) return fail(-1, "query: counter scratch missing");
+            hipLaunchKernelGGL(traverse_kernel<false>, dim3((unsigned)grid), dim3(kWave), y.lds_bytes, s, a, y);
+        }
     }
     DCIH_HIP(hipGetLastError());
     if (ev) (void)hipEventRecord(ev[1], s);

@@ -39,6 +39,7 @@ __device__ inline unsigned long long pack_key(float key, uint32_t pos) {
 template <bool FINAL>
 __global__ void segsort_tile_kernel(const float* __restrict__ keys, SegGeom g,
                                     float* __restrict__ skeys, int32_t* __restrict__ sids,
+                                    uint32_t* __restrict__ inv, uint16_t* __restrict__ lids,
                                     unsigned long long* __restrict__ packed, int np2) {
     extern __shared__ unsigned long long s[];
     const int64_t flat = blockIdx.x;
@@ -60,9 +61,31 @@ __global__ void segsort_tile_kernel(const float* __restrict__ keys, SegGeom g,
         if (FINAL) {
             skeys[base + j] = ord2f((uint32_t)(w >> 32));
             sids[base + j] = (int32_t)(off + (uint32_t)w);
+            if (lids) lids[base + j] = (uint16_t)(uint32_t)w;
         } else {
             packed[base + j] = w;
         }
+    }
+    if (FINAL && inv) {
+        // inverse permutation inv[point] = position of the point inside its
+        // sorted slice, transposed through LDS so the global write is coalesced.
+        // The position table overlays the sorted words, so each thread first
+        // pulls its words' low halves into registers.
+        uint32_t local[kTileCap / 1024];
+#pragma unroll
+        for (int r = 0; r < kTileCap / 1024; r++) {
+            const int j = threadIdx.x + r * blockDim.x;
+            local[r] = j < m ? (uint32_t)s[j] - (uint32_t)t0 : 0u;
+        }
+        __syncthreads();
+        uint32_t* pos_of = reinterpret_cast<uint32_t*>(s);
+#pragma unroll
+        for (int r = 0; r < kTileCap / 1024; r++) {
+            const int j = threadIdx.x + r * blockDim.x;
+            if (j < m) pos_of[local[r]] = (uint32_t)j;
+        }
+        __syncthreads();
+        for (int j = threadIdx.x; j < m; j += blockDim.x) inv[base + j] = pos_of[j];
     }
 }
 
@@ -110,13 +133,17 @@ __global__ __launch_bounds__(kMergeThreads) void segsort_merge_kernel(
 
 __global__ void segsort_unpack_kernel(const unsigned long long* __restrict__ packed,
                                       int64_t total, int64_t n, int64_t ppb,
-                                      float* __restrict__ skeys, int32_t* __restrict__ sids) {
+                                      float* __restrict__ skeys, int32_t* __restrict__ sids,
+                                      uint32_t* __restrict__ inv, uint16_t* __restrict__ lids) {
     const int64_t stride = (int64_t)gridDim.x * blockDim.x;
     for (int64_t e = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; e < total; e += stride) {
         const unsigned long long w = packed[e];
         const int64_t col = e % n;
+        const int64_t off = (col / ppb) * ppb;
         skeys[e] = ord2f((uint32_t)(w >> 32));
-        sids[e] = (int32_t)((col / ppb) * ppb + (uint32_t)w);
+        sids[e] = (int32_t)(off + (uint32_t)w);
+        if (inv) inv[e - col + off + (uint32_t)w] = (uint32_t)(col - off);
+        if (lids) lids[e] = (uint16_t)(uint32_t)w;
     }
 }
 
@@ -133,7 +160,8 @@ static int next_pow2(int v) {
 }
 
 int segsort(const float* d_keys, int num_indices, int64_t n, int block_size,
-            float* d_skeys, int32_t* d_sids, void* d_tmp, hipStream_t s) {
+            float* d_skeys, int32_t* d_sids, uint32_t* d_inv, uint16_t* d_lids, void* d_tmp,
+            hipStream_t s) {
     if (n <= 0) return 0;
     SegGeom g;
     g.n = n;
@@ -141,6 +169,7 @@ int segsort(const float* d_keys, int num_indices, int64_t n, int block_size,
     g.ppb = (n + block_size - 1) / block_size;
     g.tiles = (int)((g.ppb + kTileCap - 1) / kTileCap);
     const int np2 = next_pow2((int)min((int64_t)kTileCap, g.ppb));
+    // at most kTileCap / 1024 elements per thread (the inverse-permutation pass relies on it)
     const int threads = max(64, min(1024, np2 / 2));
     const size_t lds = (size_t)np2 * sizeof(unsigned long long);
     const int64_t blocks = (int64_t)num_indices * g.B * g.tiles;
@@ -159,7 +188,7 @@ int segsort(const float* d_keys, int num_indices, int64_t n, int block_size,
 
     if (g.tiles == 1) {
         hipLaunchKernelGGL(segsort_tile_kernel<true>, dim3((unsigned)blocks), dim3(threads), lds, s,
-                           d_keys, g, d_skeys, d_sids, (unsigned long long*)nullptr, np2);
+                           d_keys, g, d_skeys, d_sids, d_inv, d_lids, (unsigned long long*)nullptr, np2);
         DCIH_HIP(hipGetLastError());
         return 0;
     }
@@ -167,7 +196,7 @@ int segsort(const float* d_keys, int num_indices, int64_t n, int block_size,
     unsigned long long* bufA = (unsigned long long*)d_tmp;
     unsigned long long* bufB = bufA + (size_t)num_indices * n;
     hipLaunchKernelGGL(segsort_tile_kernel<false>, dim3((unsigned)blocks), dim3(threads), lds, s,
-                       d_keys, g, (float*)nullptr, (int32_t*)nullptr, bufA, np2);
+                       d_keys, g, (float*)nullptr, (int32_t*)nullptr, (uint32_t*)nullptr, (uint16_t*)nullptr, bufA, np2);
     const int chunks = (int)((g.ppb + kMergeChunk - 1) / kMergeChunk);
     const int64_t mblocks = (int64_t)num_indices * g.B * chunks;
     if (mblocks > 0x7fffffffLL) return fail(-1, "segsort: too many merge chunks for one launch");
@@ -179,7 +208,7 @@ int segsort(const float* d_keys, int num_indices, int64_t n, int block_size,
     const int64_t total = (int64_t)num_indices * n;
     const int ublocks = (int)min((int64_t)65536, (total + 255) / 256);
     hipLaunchKernelGGL(segsort_unpack_kernel, dim3(ublocks), dim3(256), 0, s,
-                       bufA, total, n, g.ppb, d_skeys, d_sids);
+                       bufA, total, n, g.ppb, d_skeys, d_sids, d_inv, d_lids);
     DCIH_HIP(hipGetLastError());
     return 0;
 }

@@ -1,0 +1,746 @@
+// Batch ("epoch") traversal: one workgroup per (query, partition), every lane
+// streaming index entries.
+//
+// Computes exactly what the step-by-step loop of
+// dci_query_single_point_by_block (src/dci_cuda_kernel.cu:401-626) computes,
+// without executing it step by step.  What makes that possible:
+//
+//  * Inside one simple index the windows returned by dci_next_closest_proj
+//    (:250-273) form two streams (left, right of the query position) whose
+//    priorities (:572-590) never decrease, merged nearest-first, ties to the
+//    left.  One composite index pops its L simple indices nearest-first, ties
+//    to the lowest simple index (:466-478).  So composite m consumes ALL its
+//    windows in ascending (priority, simple index, own order), window number r
+//    of that order is visited at outer step r, and "every window with priority
+//    below rho" is always a prefix of the traversal.
+//  * A point is promoted by composite m at the step of the LAST of the L
+//    windows that hold it; it is a candidate at its earliest (step, m) over
+//    the composites; the loop stops at the first step kk with
+//    c0(kk) >= k and (kk+1 >= outer*L or c0(kk) >= max_candidates), where c0
+//    counts promotions whose last window held the point in lane 0 (:598-607).
+//
+// An epoch picks a priority bound per composite index, finds by binary search
+// how many windows of every stream lie below it, and lets all lanes stream the
+// new index ranges (coalesced 4-byte id reads, packed LDS visit counters).  A
+// counter reaching L is a promotion; only for those few points the exact step
+// is computed: the inverse permutation gives the point's position in each of
+// the L simple indices, the farthest of its windows is the last one visited,
+// and that window's rank is a sum of 2L binary searches.  Promotions are then
+// replayed in (step, composite) order to apply the stop rule.  An epoch that
+// promotes too many points at once is undone (the same ranges are streamed
+// again, subtracting) and retried smaller.  Whatever does not fit the fixed LDS
+// tables is handed to the step-by-step kernel through a redo list, so results
+// never depend on which kernel produced them.
+#include "common.h"
+#include "kernels.h"
+
+namespace dcih {
+
+namespace {
+
+constexpr int kPromoCap = 256;      // promotions one epoch may produce
+constexpr int kPromoMax = 96;       // above this an epoch is undone and halved
+constexpr int kMaxEpochs = 100000;
+constexpr uint32_t kInfBits = 0x7f800000u;
+
+enum Misc {   // 32-bit scalars shared by the workgroup; kStreamedLo must stay 8-byte aligned
+    kPromoCount = 0, kEventCount, kAccCount, kFail, kStop, kC0, kStopStepLo, kStopStepHi,
+    kArmedLo, kArmedHi, kStreamedLo, kStreamedHi, kArmed, kNumCand, kTopN, kProbes, kMiscWords
+};
+
+struct BlockLayout {
+    int cbits, wpc, seen_words, counter_words;
+    int off_idx;      // per simple index: p, qp            (2 * I words)
+    int off_stream;   // per stream: consumed, previous, total, range lo/hi, chunks, pos0, prefix (9 * 2I + 1 words, incl. the stride)
+    int off_chunk0;   // per stream: global index of its first 16-byte chunk (2I 64-bit words)
+    int off_comp;     // per composite: rho bits, K, active, previous K (4 * M words)
+    int off_q;        // query row
+    int off_promo, off_events, off_acc, off_sort, off_cnt;
+    int event_cap;    // promotions waiting for the other composites (= accepted candidates per replay)
+    int sort_cap;     // power of two >= kcap + event_cap: top-k plus one batch of candidates
+    size_t lds_bytes;
+};
+
+__host__ __device__ inline int counter_bits_of(int L) {
+    return L <= 15 ? 4 : (L <= 255 ? 8 : (L <= 65535 ? 16 : 32));
+}
+
+BlockLayout make_block_layout(const QueryArgs& a) {
+    BlockLayout y;
+    const int I = a.M * a.L;
+    y.cbits = counter_bits_of(a.L);
+    const int64_t fpw = 32 / y.cbits;
+    y.wpc = (int)((a.ppb + fpw - 1) / fpw);
+    y.seen_words = (int)((a.ppb + 31) / 32);
+    y.counter_words = a.M * y.wpc + y.seen_words;
+    int o = kMiscWords * 4;
+    y.off_idx = o;      o += 2 * I * 4;
+    y.off_stream = o;   o += (9 * 2 * I + 2) * 4;
+    o = (o + 7) & ~7;
+    y.off_chunk0 = o;   o += 2 * I * 8;
+    y.off_comp = o;     o += 4 * a.M * 4;
+    y.off_q = o;        o += ((a.dim + 3) & ~3) * 4;
+    // small tables keep more workgroups resident per CU; an item that overflows them
+    // is redone by the step-by-step kernel
+    y.event_cap = 512;
+    y.sort_cap = 2;
+    while (y.sort_cap < a.kcap + y.event_cap) y.sort_cap <<= 1;
+    y.off_promo = o;    o += kPromoCap * 4;
+    y.off_acc = o;      o += y.event_cap * 4;
+    o = (o + 15) & ~15;
+    y.off_events = o;   o += y.event_cap * 8;
+    y.off_sort = o;     o += y.sort_cap * 8;
+    y.off_cnt = o;
+    y.lds_bytes = (size_t)o + (size_t)y.counter_words * 4;
+    return y;
+}
+
+struct Stream {          // one side of one simple index within the partition
+    const float* key;    // sorted keys of the slice
+    int n, T, p, side;   // side: 0 = left of the query position, 1 = right
+    float q;
+};
+
+// Priority of window j of a stream: |key[clamped start] - q| (:572-590).
+__device__ inline uint32_t stream_prio_bits(const Stream& s, int j) {
+    const int pos = s.side ? min(s.p + 1 + j * s.T, s.n - 1) : max(s.p - s.T + 1 - j * s.T, 0);
+    return __builtin_bit_cast(uint32_t, fabsf(s.key[pos] - s.q));
+}
+
+// Number of windows j in [lo, hi) of the stream with priority < x (strict) or
+// <= x, given that the predicate is monotone in j.
+__device__ inline int count_below(const Stream& s, uint32_t x, bool strict, int lo, int hi,
+                                  uint32_t& probes) {
+    while (lo < hi) {
+        const int mid = (lo + hi) >> 1;
+        const uint32_t v = stream_prio_bits(s, mid);
+        probes++;
+        if (strict ? v < x : v <= x) lo = mid + 1; else hi = mid;
+    }
+    return lo;
+}
+
+// Windows in a stream: right NR = floor((n+T-3-p)/T)+1 (0 if negative), left
+// NL = ceil((p+1)/T); from the bounds of dci_next_closest_proj (:254-263).
+__device__ inline int stream_windows(int n, int T, int p, int side) {
+    if (side) {
+        const int v = n + T - 3 - p;
+        return v < 0 ? 0 : v / T + 1;
+    }
+    return (p + T) / T;   // ceil((p + 1) / T)
+}
+
+// Index positions [a, b) covered by windows [c0, c1) of a stream.
+__device__ inline void stream_range(int n, int T, int p, int side, int c0, int c1, int& a, int& b) {
+    if (side) {
+        a = min((int64_t)n, (int64_t)p + 1 + (int64_t)c0 * T);
+        b = min((int64_t)n, (int64_t)p + 1 + (int64_t)c1 * T);
+    } else {
+        a = max((int64_t)0, (int64_t)p + 1 - (int64_t)c1 * T);
+        b = max((int64_t)0, (int64_t)p + 1 - (int64_t)c0 * T);
+    }
+}
+
+__device__ inline unsigned long long pack_event(uint32_t time, int m, bool lane0, uint32_t local) {
+    return ((unsigned long long)time << 32) | ((unsigned long long)m << 26) |
+           ((unsigned long long)(lane0 ? 1u : 0u) << 25) | local;
+}
+
+template <int NT, int CBITS>
+__global__ __launch_bounds__(NT) void traverse_block_kernel(QueryArgs a, BlockLayout y) {
+    constexpr uint32_t kFpw = 32 / CBITS;                       // counters per 32-bit word
+    constexpr int kFshift = CBITS == 4 ? 3 : 2;                 // log2(kFpw)
+    constexpr uint32_t kCmask = (1u << CBITS) - 1u;
+    extern __shared__ __align__(16) unsigned char smem[];
+    uint32_t* misc = reinterpret_cast<uint32_t*>(smem);
+    int* s_p = reinterpret_cast<int*>(smem + y.off_idx);
+    float* s_qp = reinterpret_cast<float*>(s_p + a.M * a.L);
+    int* s_c = reinterpret_cast<int*>(smem + y.off_stream);          // windows consumed
+    int* s_cprev = s_c + 2 * a.M * a.L;                               // ... at epoch start
+    int* s_ns = s_cprev + 2 * a.M * a.L;                              // windows in the stream
+    int* s_ra = s_ns + 2 * a.M * a.L;                                 // epoch's position range [ra, rb)
+    int* s_rb = s_ra + 2 * a.M * a.L;
+    int* s_nch = s_rb + 2 * a.M * a.L;                                // 16-byte chunks the range touches
+    int* s_pos0 = s_nch + 2 * a.M * a.L;                              // position of the first chunk's first id
+    int* s_stride = s_pos0 + 2 * a.M * a.L;                           // windows to try next epoch
+    int* s_pref = s_stride + 2 * a.M * a.L;                           // whole-chunk prefix sums (2I + 1)
+    long long* s_chunk0 = reinterpret_cast<long long*>(smem + y.off_chunk0);
+    uint32_t* s_rho = reinterpret_cast<uint32_t*>(smem + y.off_comp); // per composite
+    uint32_t* s_K = s_rho + a.M;
+    uint32_t* s_active = s_K + a.M;
+    uint32_t* s_Kprev = s_active + a.M;
+    float* s_q = reinterpret_cast<float*>(smem + y.off_q);
+    uint32_t* promo = reinterpret_cast<uint32_t*>(smem + y.off_promo);
+    uint32_t* acc = reinterpret_cast<uint32_t*>(smem + y.off_acc);
+    unsigned long long* events = reinterpret_cast<unsigned long long*>(smem + y.off_events);
+    unsigned long long* sortbuf = reinterpret_cast<unsigned long long*>(smem + y.off_sort);
+    uint32_t* cnt = reinterpret_cast<uint32_t*>(smem + y.off_cnt);
+    uint32_t* seen = cnt + (size_t)a.M * y.wpc;
+
+    const int tid = threadIdx.x;
+    const int lane = tid & (kWave - 1);
+    const int wave = tid / kWave;
+    constexpr int kWaves = NT / kWave;
+    // optional phase profile: thread 0 adds the 100 MHz ticks each phase took
+    unsigned long long tick = a.phase_ticks ? wall_clock64() : 0ull;
+    auto phase = [&](int which) {
+        if (a.phase_ticks && tid == 0) {
+            const unsigned long long now = wall_clock64();
+            atomicAdd(&a.phase_ticks[which], now - tick);
+            tick = now;
+        }
+    };
+    const int I = a.M * a.L;
+    const int S = 2 * I;                       // streams
+    const uint32_t Lm1 = (uint32_t)a.L - 1u;
+
+    const int64_t item = blockIdx.x;
+    const int b = (int)(item % a.B);
+    const int qi = (int)(item / a.B);
+    const int64_t off = (int64_t)b * a.ppb;
+    const int n = (int)min(a.N - off, a.ppb);
+    unsigned long long* part_out = a.part + item * a.kcap;
+    if (n <= 0) {
+        for (int j = tid; j < a.kcap; j += NT) part_out[j] = ~0ull;
+        return;
+    }
+    const int T = a.T;
+
+    // ---- set-up ---------------------------------------------------------------
+    for (int w = tid; w < y.counter_words; w += NT) cnt[w] = 0;
+    for (int j = tid; j < a.dim; j += NT) s_q[j] = a.query[(int64_t)qi * a.dim + j];
+    if (tid < kMiscWords) misc[tid] = 0;
+    uint32_t probes = 0;
+    if (tid < I) {      // positioning search (:279-297)
+        const float* key = a.skeys + (int64_t)tid * a.N + off;
+        const float qp = a.qproj[(int64_t)tid * a.nq + qi];
+        int lo = 0, hi = n;    // first position whose key is not below qp
+        while (lo < hi) {
+            const int mid = (lo + hi) >> 1;
+            probes++;
+            if (key[mid] < qp) lo = mid + 1; else hi = mid;
+        }
+        const int p = lo - 1;
+        s_p[tid] = p;
+        s_qp[tid] = qp;
+        for (int side = 0; side < 2; side++) {
+            s_ns[2 * tid + side] = stream_windows(n, T, p, side);
+            s_c[2 * tid + side] = 0;
+        }
+    }
+    __syncthreads();
+    // Stride of an epoch, in windows, per stream: starts at 1/128 of the longest
+    // stream; afterwards each stream's stride follows what it consumed last time
+    // (its local density), scaled so that every composite lands on the same step
+    // count: a composite left behind would keep the promotions of the others
+    // waiting.  The total doubles from epoch to epoch until one has to be undone.
+    {
+        int first = 4;
+        for (int s = 0; s < S; s++) first = max(first, s_ns[s] / 128);
+        if (tid < S) s_stride[tid] = first;
+        if (tid < a.M) s_Kprev[tid] = 0;
+    }
+    __syncthreads();
+    phase(0);
+
+    auto load_stream = [&](int s) {
+        Stream st;
+        const int i = s >> 1;
+        st.key = a.skeys + (int64_t)i * a.N + off;
+        st.n = n; st.T = T; st.p = s_p[i]; st.side = s & 1; st.q = s_qp[i];
+        return st;
+    };
+    // Adds (or, for undo, removes) the visits of windows [cprev, c) of all streams.
+    // The loop is bound by vector-ALU issue (about 8 instructions and one LDS
+    // atomic per visit), so it reads partition-relative 16-bit ids, eight per
+    // aligned 16-byte chunk, and keeps per-visit work to shift / mask / atomic /
+    // compare with compile-time field widths.  The whole-chunk interior of every
+    // stream's range is laid end to end: consecutive threads read consecutive
+    // chunks whatever stream they belong to, several reads in flight each.  The
+    // one or two partial chunks at the ends of a range are handled separately
+    // with masks.  Returns the entries streamed (same value on every thread).
+    auto visit = [&](uint32_t* __restrict__ mcnt, uint32_t local, int m, bool undo) {
+        const uint32_t sh = (local & (kFpw - 1u)) * CBITS;
+        if (undo) {
+            atomicSub(&mcnt[local >> kFshift], 1u << sh);
+        } else {
+            const uint32_t old = atomicAdd(&mcnt[local >> kFshift], 1u << sh);
+            if (((old >> sh) & kCmask) == Lm1) {
+                const uint32_t slot = atomicAdd(&misc[kPromoCount], 1u);
+                if (slot < (uint32_t)kPromoCap) promo[slot] = local | ((uint32_t)m << 26);
+            }
+        }
+    };
+    auto stream_epoch = [&](bool undo) {
+        constexpr int kUnroll = 4;
+        if (tid < S) {
+            const int i = tid >> 1;
+            int ra, rb;
+            stream_range(n, T, s_p[i], tid & 1, s_cprev[tid], s_c[tid], ra, rb);
+            s_ra[tid] = ra; s_rb[tid] = rb;
+            const int64_t base_idx = (int64_t)i * a.N + off;
+            const int64_t c_first = (base_idx + ra) >> 3;            // chunk holding position ra
+            const int64_t c_end = (base_idx + rb + 7) >> 3;          // one past the chunk holding rb-1
+            s_chunk0[tid] = c_first;
+            s_nch[tid] = rb > ra ? (int)(c_end - c_first) : 0;
+            s_pos0[tid] = (int)((c_first << 3) - base_idx);          // position of that chunk's first id
+        }
+        __syncthreads();
+        if (tid == 0) {          // prefix over the interior (whole) chunks of every stream
+            int acc_chunks = 0;
+            for (int s = 0; s < S; s++) {
+                s_pref[s] = acc_chunks;
+                acc_chunks += max(0, s_nch[s] - 2);
+            }
+            s_pref[S] = acc_chunks;
+        }
+        __syncthreads();
+        const uint4* all = reinterpret_cast<const uint4*>(a.lids);
+        // partial chunks: the first and the last chunk of every range
+        if (tid < 2 * S) {
+            const int s = tid >> 1;
+            const int nch = s_nch[s];
+            const int which = tid & 1;                 // 0 = first chunk, 1 = last chunk
+            if (nch > which) {
+                const int cidx = which ? nch - 1 : 0;
+                const uint4 r = all[s_chunk0[s] + cidx];
+                const int pos0 = s_pos0[s] + (cidx << 3);
+                const int ra = s_ra[s], rb = s_rb[s];
+                const int m = (s >> 1) / a.L;
+                uint32_t* mcnt = cnt + (size_t)m * y.wpc;
+                const uint32_t w[4] = {r.x, r.y, r.z, r.w};
+#pragma unroll
+                for (int e = 0; e < 8; e++) {
+                    const int pos = pos0 + e;
+                    if (pos >= ra && pos < rb) visit(mcnt, (w[e >> 1] >> ((e & 1) * 16)) & 0xffffu, m, undo);
+                }
+            }
+        }
+        // whole chunks
+        const int total = s_pref[S];
+        int cur = 0;
+        for (int g0 = 0; g0 < total; g0 += NT * kUnroll) {
+            uint4 r[kUnroll];
+            int sreg[kUnroll];
+#pragma unroll
+            for (int u = 0; u < kUnroll; u++) {
+                const int g = g0 + u * NT + tid;
+                sreg[u] = -1;
+                if (g < total) {
+                    while (g >= s_pref[cur + 1]) cur++;
+                    sreg[u] = cur;
+                    r[u] = all[s_chunk0[cur] + 1 + (g - s_pref[cur])];
+                }
+            }
+            if (undo) {
+#pragma unroll
+                for (int u = 0; u < kUnroll; u++) {
+                    if (sreg[u] < 0) continue;
+                    uint32_t* mcnt = cnt + (size_t)((sreg[u] >> 1) / a.L) * y.wpc;
+                    const uint32_t w[4] = {r[u].x, r[u].y, r[u].z, r[u].w};
+#pragma unroll
+                    for (int e = 0; e < 8; e++) {
+                        const uint32_t local = (w[e >> 1] >> ((e & 1) * 16)) & 0xffffu;
+                        atomicSub(&mcnt[local >> kFshift], 1u << ((local & (kFpw - 1u)) * CBITS));
+                    }
+                }
+            } else {
+                // all atomics of the batch first, then the (rare) promotions: a compare
+                // right behind each returning atomic would serialise on LDS latency
+                uint32_t old[kUnroll][8];
+#pragma unroll
+                for (int u = 0; u < kUnroll; u++) {
+                    if (sreg[u] < 0) continue;
+                    uint32_t* mcnt = cnt + (size_t)((sreg[u] >> 1) / a.L) * y.wpc;
+                    const uint32_t w[4] = {r[u].x, r[u].y, r[u].z, r[u].w};
+#pragma unroll
+                    for (int e = 0; e < 8; e++) {
+                        const uint32_t local = (w[e >> 1] >> ((e & 1) * 16)) & 0xffffu;
+                        old[u][e] = atomicAdd(&mcnt[local >> kFshift], 1u << ((local & (kFpw - 1u)) * CBITS));
+                    }
+                }
+#pragma unroll
+                for (int u = 0; u < kUnroll; u++) {
+                    if (sreg[u] < 0) continue;
+                    const uint32_t w[4] = {r[u].x, r[u].y, r[u].z, r[u].w};
+#pragma unroll
+                    for (int e = 0; e < 8; e++) {
+                        const uint32_t local = (w[e >> 1] >> ((e & 1) * 16)) & 0xffffu;
+                        if (((old[u][e] >> ((local & (kFpw - 1u)) * CBITS)) & kCmask) == Lm1) {
+                            const uint32_t slot = atomicAdd(&misc[kPromoCount], 1u);
+                            if (slot < (uint32_t)kPromoCap)
+                                promo[slot] = local | ((uint32_t)((sreg[u] >> 1) / a.L) << 26);
+                        }
+                    }
+                }
+            }
+        }
+        unsigned long long streamed = 0;
+        for (int s = 0; s < S; s++) streamed += (unsigned long long)max(0, s_rb[s] - s_ra[s]);
+        return streamed;
+    };
+
+    unsigned long long streamed = 0;     // entries streamed so far (same on every thread)
+    bool shrunk = false;
+    int epoch = 0;
+    for (; epoch < kMaxEpochs; epoch++) {
+        // ---- 1. priority bound per composite ------------------------------------
+        if (tid < a.M) { s_rho[tid] = kInfBits; s_K[tid] = 0; s_active[tid] = 0; }
+        __syncthreads();
+        if (tid < S) {
+            const int c = s_c[tid], ns = s_ns[tid];
+            s_cprev[tid] = c;
+            if (c < ns) {
+                const int m = (tid >> 1) / a.L;
+                const Stream st = load_stream(tid);
+                const int64_t jp = min((int64_t)c + s_stride[tid], (int64_t)ns) - 1;
+                probes++;
+                atomicMin(&s_rho[m], stream_prio_bits(st, (int)jp));
+                atomicAdd(&s_active[m], 1u);
+            }
+        }
+        __syncthreads();
+        phase(1);
+        // ---- 2. how far each stream goes: all windows with priority <= bound ----
+        if (tid < S) {
+            const int c = s_c[tid], ns = s_ns[tid];
+            const int m = (tid >> 1) / a.L;
+            const uint32_t rho = s_rho[m];
+            int cn = c;
+            if (c < ns && rho < kInfBits) {
+                const Stream st = load_stream(tid);
+                // gallop to an upper bound, then bisect
+                int64_t step = s_stride[tid];
+                int lo = c, hi = (int)min((int64_t)ns, (int64_t)c + step);
+                while (hi < ns) {
+                    probes++;
+                    if (stream_prio_bits(st, hi - 1) <= rho) {
+                        lo = hi; step *= 2; hi = (int)min((int64_t)ns, (int64_t)hi + step);
+                    } else break;
+                }
+                cn = count_below(st, rho, false, lo, hi, probes);
+            } else if (c < ns) {
+                cn = ns;     // NaN priorities: take the rest so the epoch loop ends
+            }
+            s_c[tid] = cn;
+            atomicAdd(&s_K[m], (uint32_t)cn);
+        }
+        __syncthreads();
+        bool all_done = true;
+        for (int m = 0; m < a.M; m++) all_done = all_done && s_active[m] == 0;
+        if (all_done) break;      // every stream was already exhausted before this epoch
+        phase(2);
+
+        // ---- 3. stream the new ranges ---------------------------------------------
+        streamed += stream_epoch(false);
+        __syncthreads();
+        phase(3);
+        const uint32_t np = misc[kPromoCount];
+        // too many promotions at once (or no room left beside the ones still waiting
+        // for the other composites): take the epoch back and retry with half the stride
+        if (np > (uint32_t)kPromoMax || misc[kEventCount] + np > (uint32_t)y.event_cap) {
+            bool minimal = true;
+            for (int s2 = 0; s2 < S; s2++) minimal = minimal && s_stride[s2] <= 1;
+            if (minimal && np <= (uint32_t)kPromoCap && misc[kEventCount] + np <= (uint32_t)y.event_cap) {
+                // cannot go smaller; the tables still hold it
+            } else if (minimal) {
+                if (tid == 0) misc[kFail] = 2;
+                __syncthreads();
+                break;
+            } else {
+                streamed += stream_epoch(true);
+                __syncthreads();
+                if (tid < S) s_c[tid] = s_cprev[tid];
+                if (tid < S) s_stride[tid] = max(1, s_stride[tid] / 2);
+                if (tid == 0) misc[kPromoCount] = 0;
+                shrunk = true;
+                __syncthreads();
+                phase(4);
+                continue;
+            }
+        }
+
+        // ---- 4. exact step of every promotion -----------------------------------
+        {
+            constexpr int kGroup = 32;
+            const int gl = tid & (kGroup - 1);
+            const int group = tid / kGroup;
+            for (uint32_t pi = group; pi < np; pi += NT / kGroup) {
+                const uint32_t pr = promo[pi];
+                const uint32_t local = pr & 0x3ffffffu;
+                const int m = (int)(pr >> 26);
+                // farthest of the L windows that hold the point = the last one visited
+                uint32_t w_bits = 0;
+                int w_h = -1, w_side = 0, w_j = 0, w_t = 0;
+                for (int h = gl; h < a.L; h += kGroup) {
+                    const int i = m * a.L + h;
+                    const int pos = (int)a.inv[(int64_t)i * a.N + off + local];
+                    const int p = s_p[i];
+                    const float* key = a.skeys + (int64_t)i * a.N + off;
+                    int side, j, t, kp;
+                    if (pos > p) {
+                        const int d = pos - (p + 1);
+                        side = 1; j = d / T; t = d - j * T; kp = p + 1 + j * T;
+                    } else {
+                        const int d = p - pos;
+                        side = 0; j = d / T;
+                        const int start = p - T + 1 - j * T;
+                        t = pos - start; kp = max(start, 0);
+                    }
+                    probes++;
+                    const uint32_t bits = __builtin_bit_cast(uint32_t, fabsf(key[kp] - s_qp[i]));
+                    if (w_h < 0 || bits >= w_bits) { w_bits = bits; w_h = h; w_side = side; w_j = j; w_t = t; }
+                }
+                for (int o = kGroup / 2; o > 0; o >>= 1) {
+                    const uint32_t ob = (uint32_t)__shfl_xor((int)w_bits, o, kGroup);
+                    const int oh = __shfl_xor(w_h, o, kGroup);
+                    const int os = __shfl_xor(w_side, o, kGroup);
+                    const int oj = __shfl_xor(w_j, o, kGroup);
+                    const int ot = __shfl_xor(w_t, o, kGroup);
+                    const bool take = oh >= 0 && (w_h < 0 || ob > w_bits || (ob == w_bits && oh > w_h));
+                    if (take) { w_bits = ob; w_h = oh; w_side = os; w_j = oj; w_t = ot; }
+                }
+                // rank of that window = windows of the composite ordered before it
+                uint32_t rank = 0;
+                for (int s2 = gl; s2 < 2 * a.L; s2 += kGroup) {
+                    const int h2 = s2 >> 1, side2 = s2 & 1;
+                    const int sidx = 2 * (m * a.L + h2) + side2;
+                    const int lo = s_cprev[sidx], hi = s_c[sidx];
+                    int c;
+                    if (h2 == w_h) {
+                        const bool corner = s_p[m * a.L + h2] == n - 1 && T >= 2;  // ghost window first
+                        if (side2 == w_side) c = w_j;
+                        else if (corner) c = w_side ? 0 : s_ns[sidx];
+                        else c = count_below(load_stream(sidx), w_bits, w_side == 0, lo, hi, probes);
+                    } else {
+                        c = count_below(load_stream(sidx), w_bits, h2 > w_h, lo, hi, probes);
+                    }
+                    rank += (uint32_t)c;
+                }
+                for (int o = kGroup / 2; o > 0; o >>= 1) rank += (uint32_t)__shfl_xor((int)rank, o, kGroup);
+                if (gl == 0) {
+                    const uint32_t slot = atomicAdd(&misc[kEventCount], 1u);
+                    if (slot < (uint32_t)y.event_cap) events[slot] = pack_event(rank, m, w_t == 0, local);
+                    else misc[kFail] = 3;
+                }
+            }
+        }
+        __syncthreads();
+        phase(5);
+        if (misc[kFail]) break;
+
+        // ---- 5. replay promotions in (step, composite) order ----------------------
+        const int ne = (int)misc[kEventCount];
+        unsigned long long H = ~0ull;        // steps below H are complete for every composite
+        for (int m = 0; m < a.M; m++) {
+            bool exhausted = true;
+            for (int h = 0; h < 2 * a.L; h++) {
+                const int sidx = 2 * m * a.L + h;
+                exhausted = exhausted && s_c[sidx] >= s_ns[sidx];
+            }
+            if (!exhausted) H = min(H, (unsigned long long)s_K[m]);
+        }
+        if (ne > 0) {
+            int np2 = 2;
+            while (np2 < ne) np2 <<= 1;
+            for (int j = ne + tid; j < np2; j += NT) events[j] = ~0ull;
+            bitonic_sort_u64(events, np2);
+        }
+        if (tid == 0) {
+            long long c0 = (long long)misc[kC0];
+            bool armed = misc[kArmed] != 0;
+            unsigned long long t_armed = ((unsigned long long)misc[kArmedHi] << 32) | misc[kArmedLo];
+            uint32_t nacc = misc[kAccCount];
+            uint32_t ncand = misc[kNumCand];
+            bool stop = false;
+            unsigned long long kk_star = 0;
+            const unsigned long long last_needed = a.stop_at > 0 ? (unsigned long long)(a.stop_at - 1) : 0ull;
+            int idx = 0;
+            while (idx < ne) {
+                const unsigned long long t = events[idx] >> 32;
+                if (t >= H) break;
+                if (armed) {
+                    const unsigned long long cand = max(t_armed, last_needed);
+                    if (cand < t) { stop = true; kk_star = cand; break; }
+                }
+                // all events of step t
+                while (idx < ne && (events[idx] >> 32) == t) {
+                    const uint32_t e = (uint32_t)events[idx];
+                    const uint32_t local = e & 0x1ffffffu;
+                    const uint32_t bit = 1u << (local & 31);
+                    if (!(seen[local >> 5] & bit)) {
+                        seen[local >> 5] |= bit;
+                        acc[nacc++] = local;
+                        ncand++;
+                        if (e & (1u << 25)) c0++;
+                    }
+                    idx++;
+                }
+                if (c0 >= a.k) {
+                    if (!armed) { armed = true; t_armed = t; }
+                    if (c0 >= a.max_cand || (long long)(t + 1) >= a.stop_at) { stop = true; kk_star = t; break; }
+                }
+            }
+            if (!stop && armed) {
+                const unsigned long long cand = max(t_armed, last_needed);
+                if (cand < H) { stop = true; kk_star = cand; }
+            }
+            // keep what is not settled yet
+            int keep = 0;
+            if (!stop) for (; idx < ne; idx++) events[keep++] = events[idx];
+            misc[kEventCount] = (uint32_t)keep;
+            misc[kC0] = (uint32_t)c0;
+            misc[kArmed] = armed ? 1u : 0u;
+            misc[kArmedLo] = (uint32_t)t_armed; misc[kArmedHi] = (uint32_t)(t_armed >> 32);
+            misc[kAccCount] = nacc;
+            misc[kNumCand] = ncand;
+            misc[kStop] = stop ? 1u : 0u;
+            misc[kStopStepLo] = (uint32_t)kk_star; misc[kStopStepHi] = (uint32_t)(kk_star >> 32);
+            misc[kPromoCount] = 0;
+        }
+        __syncthreads();
+        phase(6);
+
+        // ---- 6. distances of the accepted candidates, merged into the top-k ---------
+        const int nacc = (int)misc[kAccCount];
+        const bool stop = misc[kStop] != 0;
+        if (nacc > 0) {
+            const int topn = (int)misc[kTopN];
+            for (int c = wave; c < nacc; c += kWaves) {
+                const int64_t pt = off + acc[c];
+                const float* row = a.data + pt * a.dim;
+                float sum = 0.f;
+                for (int j = lane; j < a.dim; j += kWave) {
+                    const float df = row[j] - s_q[j];
+                    sum = __builtin_fmaf(df, df, sum);
+                }
+                const float dist = sqrtf(wave_sum(sum));
+                if (lane == 0)
+                    sortbuf[topn + c] = ((unsigned long long)__builtin_bit_cast(uint32_t, dist) << 32) | (uint32_t)pt;
+            }
+            int np2 = 2;
+            while (np2 < topn + nacc) np2 <<= 1;
+            for (int j = topn + nacc + tid; j < np2; j += NT) sortbuf[j] = ~0ull;
+            bitonic_sort_u64(sortbuf, np2);
+            if (tid == 0) {
+                misc[kTopN] = (uint32_t)min(a.kcap, topn + nacc);
+                misc[kAccCount] = 0;
+            }
+            __syncthreads();
+        }
+        phase(7);
+        if (stop) break;
+        bool exhausted_all = true;
+        for (int s = 0; s < S; s++) exhausted_all = exhausted_all && s_c[s] >= s_ns[s];
+        if (exhausted_all) break;     // H was unbounded: everything has been replayed
+        {
+            uint32_t kmax = 0, dk_lead = 1;
+            for (int m = 0; m < a.M; m++)
+                if (s_K[m] >= kmax) { kmax = s_K[m]; dk_lead = max(1u, s_K[m] - s_Kprev[m]); }
+            const float k_target = (float)kmax + (shrunk ? 1.0f : 2.0f) * (float)dk_lead;
+            __syncthreads();
+            if (tid < S) {
+                const int m = (tid >> 1) / a.L;
+                const float dk = (float)max(1u, s_K[m] - s_Kprev[m]);
+                const float scale = fminf(16.0f, fmaxf(0.0f, k_target - (float)s_K[m]) / dk);
+                const float want = ceilf((float)max(1, s_c[tid] - s_cprev[tid]) * scale);
+                s_stride[tid] = (int)fminf(fmaxf(want, 1.0f), 16777216.0f);
+            }
+            __syncthreads();
+            if (tid < a.M) s_Kprev[tid] = s_K[tid];
+            __syncthreads();
+        }
+    }
+    __syncthreads();
+
+    if (misc[kFail] || epoch >= kMaxEpochs) {
+        // hand the item to the step-by-step kernel
+        if (a.phase_ticks && tid == 0) {
+            atomicAdd(&a.phase_ticks[10], 1ull);
+            atomicAdd(&a.phase_ticks[11 + min(3u, misc[kFail])], 1ull);
+            a.phase_ticks[15] = ((unsigned long long)item << 32) | ((unsigned long long)misc[kEventCount] << 16) | misc[kPromoCount];
+        }
+        if (tid == 0) {
+            const uint32_t slot = atomicAdd(a.redo_count, 1u);
+            a.redo_items[slot] = (int32_t)item;
+        }
+        return;
+    }
+
+    if (a.phase_ticks && tid == 0) {
+        atomicAdd(&a.phase_ticks[8], (unsigned long long)epoch + 1);
+        atomicAdd(&a.phase_ticks[9], 1ull);
+    }
+    // ---- results -------------------------------------------------------------------
+    const int topn = (int)misc[kTopN];
+    for (int j = tid; j < a.kcap; j += NT) part_out[j] = j < topn ? sortbuf[j] : ~0ull;
+    if (a.counters) {
+        for (int o = 32; o > 0; o >>= 1) probes += (uint32_t)__shfl_xor((int)probes, o, kWave);
+        if (lane == 0) atomicAdd(&misc[kProbes], probes);
+        if (tid == 0) { misc[kStreamedLo] = (uint32_t)streamed; misc[kStreamedHi] = (uint32_t)(streamed >> 32); }
+        __syncthreads();
+        if (tid == 0) {
+            unsigned long long steps;   // outer steps the loop would have run (:458, :598-609)
+            const unsigned long long bound = (unsigned long long)n * a.L * T;
+            unsigned long long maxw = 0;
+            for (int m = 0; m < a.M; m++) {
+                unsigned long long w = 0;
+                for (int h = 0; h < 2 * a.L; h++) w += (unsigned long long)s_ns[2 * m * a.L + h];
+                maxw = max(maxw, w);
+            }
+            if (misc[kStop]) {
+                steps = (((unsigned long long)misc[kStopStepHi] << 32) | misc[kStopStepLo]) + 1;
+                steps = min(steps, min(bound, maxw + 1));
+            } else {
+                steps = min(bound, maxw + 1);
+            }
+            const unsigned long long st = ((unsigned long long)misc[kStreamedHi] << 32) | misc[kStreamedLo];
+            atomicAdd(&a.counters[(int64_t)qi * 4 + 0], st);
+            atomicAdd(&a.counters[(int64_t)qi * 4 + 1], (unsigned long long)misc[kNumCand]);
+            atomicAdd(&a.counters[(int64_t)qi * 4 + 2], (unsigned long long)misc[kProbes]);
+            atomicAdd(&a.counters[(int64_t)qi * 4 + 3], steps);
+        }
+    }
+}
+
+constexpr int kBlockThreads = 256;
+
+}  // namespace
+
+bool block_traversal_supported(const QueryArgs& a, size_t* lds_bytes) {
+    const BlockLayout y = make_block_layout(a);
+    if (lds_bytes) *lds_bytes = y.lds_bytes;
+    const int I = a.M * a.L;
+    if (!a.inv || !a.lids || a.ppb > 65536) return false;
+    if (a.L > 255) return false;            // 4- and 8-bit visit counters only
+    if (4 * I > kBlockThreads || a.M > 64) return false;   // one thread per partial chunk of a stream
+    if (a.kcap > 512) return false;
+    if (a.ppb >= (1 << 25)) return false;
+    if ((int64_t)a.L * (a.ppb + 2 * (int64_t)a.T) >= 0x7fffffffLL) return false;   // steps fit 32 bits
+    if ((int64_t)a.ppb + 2 * (int64_t)a.T >= 0x7fffffffLL) return false;
+    if ((int64_t)a.nq * a.B > 0x7fffffffLL) return false;
+    return y.lds_bytes <= 160 * 1024 - 512;
+}
+
+int query_block(const QueryArgs& a, hipStream_t s) {
+    const BlockLayout y = make_block_layout(a);
+    static bool attr_done = false;
+    if (!attr_done) {
+        DCIH_HIP(hipFuncSetAttribute((const void*)traverse_block_kernel<kBlockThreads, 4>,
+                                     hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024));
+        DCIH_HIP(hipFuncSetAttribute((const void*)traverse_block_kernel<kBlockThreads, 8>,
+                                     hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024));
+        attr_done = true;
+    }
+    const int64_t items = (int64_t)a.nq * a.B;
+    if (y.cbits == 4)
+        hipLaunchKernelGGL((traverse_block_kernel<kBlockThreads, 4>), dim3((unsigned)items),
+                           dim3(kBlockThreads), y.lds_bytes, s, a, y);
+    else
+        hipLaunchKernelGGL((traverse_block_kernel<kBlockThreads, 8>), dim3((unsigned)items),
+                           dim3(kBlockThreads), y.lds_bytes, s, a, y);
+    DCIH_HIP(hipGetLastError());
+    return 0;
+}
+
+}  // namespace dcih

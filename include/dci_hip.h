@@ -49,6 +49,18 @@ enum {
     DCIH_NUM_TIMERS = 5
 };
 
+/*
+ * Options of dcih_set_option.  DCIH_OPT_TRAVERSAL picks the query kernel:
+ * 0 = automatic (the batch kernel when the shape fits its tables, else the
+ * step-by-step kernel), 1 = step-by-step kernel (one wavefront per partition,
+ * one window per step), 2 = batch kernel (one workgroup per partition, whole
+ * index ranges per epoch; errors out if the shape does not fit).  Both give the
+ * same neighbours; with the batch kernel DCIH_CTR_VISITED counts the entries it
+ * streamed (a superset of the reference's visits, it overshoots the stop step
+ * inside its last epoch) and DCIH_CTR_PROBES its own key reads.
+ */
+enum { DCIH_OPT_TRAVERSAL = 0 };
+
 /* Message for the last failing call on this thread ("" if none). */
 const char* dcih_last_error(void);
 
@@ -112,6 +124,9 @@ int dcih_query(dcih_index* h, int dim, int num_queries, const float* d_query,
  */
 int dcih_get_index(const dcih_index* h, float* h_keys, int32_t* h_ids);
 
+/* Tuning knobs (no counterpart in the reference); see the DCIH_OPT_* list. */
+int dcih_set_option(dcih_index* h, int option, int value);
+
 /*
  * Per-kernel timing with HIP events on the caller's stream (no counterpart in
  * the reference).  After dcih_profile(h, 1) every dcih_add / dcih_query
@@ -121,6 +136,15 @@ int dcih_get_index(const dcih_index* h, float* h_keys, int32_t* h_ids);
  */
 int dcih_profile(dcih_index* h, int enable);
 int dcih_last_timings(dcih_index* h, float* h_ms);
+
+/*
+ * Phase profile of the batch traversal kernel (no counterpart in the
+ * reference).  d_ticks is NULL (off) or a zeroed device array of 16 uint64 that
+ * later dcih_query calls add to: [0..7] = 100 MHz ticks one thread of every
+ * workgroup spent in set-up, bound selection, range search, streaming, undo,
+ * promotion ranking, replay, distances/top-k; [8] = epochs, [9] = workgroups.
+ */
+int dcih_phase_profile(dcih_index* h, uint64_t* d_ticks);
 
 /* Number of points currently indexed (0 when empty). */
 int64_t dcih_num_points(const dcih_index* h);
