@@ -89,6 +89,8 @@ struct dcih_index {
     int32_t* d_sids = nullptr;          // [I][n]
     uint32_t* d_inv = nullptr;          // [I][n] position of each point in its sorted slice
     uint16_t* d_lids = nullptr;         // [I][n] partition-relative ids (partitions <= 65536 points)
+    float* d_stop_hint = nullptr;       // [block_size] epoch-size hints learnt from earlier queries
+    int hint_k = 0, hint_outer = 0, hint_T = 0, hint_maxc = 0;   // query shape the hints belong to
     int traversal = 0;                  // DCIH_OPT_TRAVERSAL value
     unsigned long long* d_phase_ticks = nullptr;   // optional profile of the batch kernel
     // grow-only query workspace
@@ -130,6 +132,7 @@ int release_index(dcih_index* h) {
     if (h->d_sids) { DCIH_HIP(hipFree(h->d_sids)); h->d_sids = nullptr; }
     if (h->d_inv) { DCIH_HIP(hipFree(h->d_inv)); h->d_inv = nullptr; }
     if (h->d_lids) { DCIH_HIP(hipFree(h->d_lids)); h->d_lids = nullptr; }
+    if (h->d_stop_hint) { DCIH_HIP(hipFree(h->d_stop_hint)); h->d_stop_hint = nullptr; }
     h->d_data = nullptr;
     h->n = 0;
     h->block_size = 0;
@@ -228,9 +231,14 @@ int dcih_add(dcih_index* h, int dim, int64_t num_points, const float* d_data,
             hipMalloc(&h->d_inv, cells * sizeof(uint32_t)) != hipSuccess ||
             // +16: the traversal reads whole aligned 16-byte chunks, also at the very end
             (small_parts && hipMalloc(&h->d_lids, (cells + 16) * sizeof(uint16_t)) != hipSuccess) ||
+            hipMalloc(&h->d_stop_hint, (size_t)block_size * sizeof(float)) != hipSuccess ||
             hipMalloc(&d_keys, cells * sizeof(float)) != hipSuccess ||
             (tmp_bytes && hipMalloc(&d_tmp, tmp_bytes) != hipSuccess)) {
             rc = fail(DCIH_EHIP, "dcih_add: out of device memory");
+            break;
+        }
+        if (hipMemsetAsync(h->d_stop_hint, 0, (size_t)block_size * sizeof(float), s) != hipSuccess) {
+            rc = fail(DCIH_EHIP, "dcih_add: clearing the hint table failed");
             break;
         }
         mark(h, DCIH_T_PROJECT, 0, s);
@@ -278,6 +286,14 @@ int dcih_query(dcih_index* h, int dim, int num_queries, const float* d_query,
     a.skeys = h->d_skeys; a.sids = h->d_sids; a.inv = h->d_inv; a.lids = h->d_lids; a.data = h->d_data; a.query = d_query;
     a.mode = h->traversal; a.item_list = nullptr; a.item_count = nullptr;
     a.phase_ticks = h->d_phase_ticks;
+    // the hints describe where traversals of one query shape stop; forget them when it changes
+    if (h->hint_k != num_neighbours || h->hint_outer != num_outer_iterations ||
+        h->hint_T != thread_size || h->hint_maxc != max_num_candidates) {
+        DCIH_HIP(hipMemsetAsync(h->d_stop_hint, 0, (size_t)block_size * sizeof(float), s));
+        h->hint_k = num_neighbours; h->hint_outer = num_outer_iterations;
+        h->hint_T = thread_size; h->hint_maxc = max_num_candidates;
+    }
+    a.stop_hint = h->d_stop_hint;
     a.N = h->n;
     a.ppb = (h->n + block_size - 1) / block_size;
     a.dim = dim; a.M = h->M; a.L = h->L; a.B = block_size; a.T = thread_size;

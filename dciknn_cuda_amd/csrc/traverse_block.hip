@@ -234,9 +234,14 @@ __global__ __launch_bounds__(NT) void traverse_block_kernel(QueryArgs a, BlockLa
     // (its local density), scaled so that every composite lands on the same step
     // count: a composite left behind would keep the promotions of the others
     // waiting.  The total doubles from epoch to epoch until one has to be undone.
+    // hint = running average of the step at which earlier queries stopped in this
+    // partition; it only steers epoch sizes (first jump to 3/4 of it, then +12 %
+    // per epoch), never results.
+    const float hint = a.stop_hint ? a.stop_hint[b] : 0.0f;
     {
         int first = 4;
         for (int s = 0; s < S; s++) first = max(first, s_ns[s] / 128);
+        if (hint > 0.0f) first = max(first, (int)(0.75f * hint / (float)(2 * a.L)));
         if (tid < S) s_stride[tid] = first;
         if (tid < a.M) s_Kprev[tid] = 0;
     }
@@ -637,7 +642,9 @@ __global__ __launch_bounds__(NT) void traverse_block_kernel(QueryArgs a, BlockLa
             uint32_t kmax = 0, dk_lead = 1;
             for (int m = 0; m < a.M; m++)
                 if (s_K[m] >= kmax) { kmax = s_K[m]; dk_lead = max(1u, s_K[m] - s_Kprev[m]); }
-            const float k_target = (float)kmax + (shrunk ? 1.0f : 2.0f) * (float)dk_lead;
+            float k_target = (float)kmax + (shrunk ? 1.0f : 2.0f) * (float)dk_lead;
+            if (hint > 0.0f && !shrunk)
+                k_target = (float)kmax < 0.7f * hint ? 0.75f * hint : 1.12f * (float)kmax + (float)S;
             __syncthreads();
             if (tid < S) {
                 const int m = (tid >> 1) / a.L;
@@ -670,6 +677,11 @@ __global__ __launch_bounds__(NT) void traverse_block_kernel(QueryArgs a, BlockLa
     if (a.phase_ticks && tid == 0) {
         atomicAdd(&a.phase_ticks[8], (unsigned long long)epoch + 1);
         atomicAdd(&a.phase_ticks[9], 1ull);
+    }
+    if (a.stop_hint && tid == 0 && misc[kStop]) {
+        const float cur = (float)((((unsigned long long)misc[kStopStepHi] << 32) | misc[kStopStepLo]) + 1);
+        const float old = a.stop_hint[b];     // racy on purpose: any recent value will do
+        a.stop_hint[b] = old > 0.0f ? 0.75f * old + 0.25f * cur : cur;
     }
     // ---- results -------------------------------------------------------------------
     const int topn = (int)misc[kTopN];
