@@ -25,7 +25,7 @@ HBM_PEAK_GBS = 8000.0   # MI355X HBM3E
 # the fastest setting found with recall@k >= 0.95 on that workload.
 TUNED = {
     "c1": dict(bs=100, ts=10, outer=5000),
-    "c2": dict(bs=100, ts=10, outer=500),
+    "c2": dict(bs=32, ts=4, outer=500),
     "c3": dict(bs=1000, ts=16, outer=500),
     "c4": dict(bs=100, ts=10, outer=500),
 }
@@ -46,6 +46,12 @@ def parse():
                    help="queries in the CPU baseline sample")
     p.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     p.add_argument("--build-reps", type=int, default=3)
+    p.add_argument("--counter-queries", type=int, default=512,
+                   help="queries whose exact traversal counters are taken (step-by-step kernel)")
+    p.add_argument("--traversal", default="auto", choices=["auto", "step", "batch"])
+    p.add_argument("--copy-calibration", action="store_true",
+                   help="also run a plain 1 GiB device copy (known HBM traffic) so that "
+                        "rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE readings can be scaled")
     return p.parse_args()
 
 
@@ -98,7 +104,15 @@ def main():
     Xd, Qd = X.cuda(), Q.cuda()
     torch.cuda.synchronize()
 
-    dci = D.DCI(dim, M, L, cfg["bs"], cfg["ts"], seed=4)
+    if a.copy_calibration:
+        src = torch.empty(1 << 28, dtype=torch.float32, device="cuda").normal_()
+        dst = torch.empty_like(src)
+        for _ in range(3):
+            dst.copy_(src)      # reads 1 GiB, writes 1 GiB
+        torch.cuda.synchronize()
+        del src, dst
+
+    dci = D.DCI(dim, M, L, cfg["bs"], cfg["ts"], seed=4, traversal=a.traversal)
     lib = dci._lib
     _capi.check(lib.dcih_profile(dci._dci_inst, 1))
     tms = (_capi.ctypes.c_float * _capi.NUM_TIMERS)()
@@ -140,20 +154,35 @@ def main():
     # ---- outside the timed region: recall and traversal counters -------------
     gt = exact_knn_gpu(Xd, Qd, k)
     recall = recall_at_k(ids.long(), gt)
+    # what the kernel that was timed actually streamed / probed
     _, _, ctr = dci.query(Qd, k, cfg["outer"], return_int=True, return_counters=True)
     torch.cuda.synchronize()
+    own = ctr.double().mean(0).cpu().numpy()
+    # exact counters of the reference algorithm (identical to the oracle's: the parity
+    # tests check that) from the step-by-step kernel on a sample of the queries
+    nqc = min(nq, a.counter_queries)
+    dci.set_traversal("step")
+    _, _, ctr = dci.query(Qd[:nqc].contiguous(), k, cfg["outer"], return_int=True, return_counters=True)
+    torch.cuda.synchronize()
+    dci.set_traversal(a.traversal)
     cm = ctr.double().mean(0).cpu().numpy()
     V, C, S, steps_q = (float(v) for v in cm)
 
-    # algorithmic bytes of the traversal kernel per query: the query row, one
-    # key per search probe, one 4-byte id per visited entry, one data row per
-    # promoted point, k results.
-    bytes_per_query = 4 * dim + 4 * S + 4 * V + 4 * dim * C + 8 * k
+    # Algorithmic bytes per query as the roofline contract defines them for this
+    # path: query row, 8 bytes (key, id) per search probe and per visited entry,
+    # one data row per promoted point, k results.  This engine stores ids apart
+    # from keys, 2 bytes each, and reads keys only where priorities are needed, so
+    # the bytes it has to move for the same work are far fewer: own_layout below.
+    bytes_per_query = 4 * dim + 8 * S + 8 * V + 4 * dim * C + 8 * k
+    bytes_own = 4 * dim + 4 * float(own[2]) + 2 * float(own[0]) + 4 * dim * C + 8 * k + 4 * M * L * C
     trav_avg_ms = float(np.mean(trav_ms))
     achieved = bytes_per_query * nq / (trav_avg_ms * 1e-3) / 1e9
-    roofline = dict(bound="hbm", kernel="traverse_kernel", achieved=achieved, peak=HBM_PEAK_GBS,
+    kernel = "traverse_kernel" if a.traversal == "step" else "traverse_block_kernel"
+    roofline = dict(bound="hbm", kernel=kernel, achieved=achieved, peak=HBM_PEAK_GBS,
                     unit="GB/s", frac=achieved / HBM_PEAK_GBS, traffic=None,
-                    bytes_per_launch=bytes_per_query * nq, avg_launch_ms=trav_avg_ms)
+                    bytes_per_launch=bytes_per_query * nq, avg_launch_ms=trav_avg_ms,
+                    own_layout_bytes_per_launch=bytes_own * nq,
+                    own_layout_gbs=bytes_own * nq / (trav_avg_ms * 1e-3) / 1e9)
     build_bytes_proj = 4.0 * N * (dim + I)
     build_bytes_sort = 12.0 * N * I
     build = dict(points_per_s=N / build_wall, wall_ms=build_wall * 1e3,
@@ -169,8 +198,8 @@ def main():
         from oracle import dci_oracle as O
         P = dci.directions.numpy()
         Xn = X.numpy()
-        nqc = min(nq, a.cpu_queries)
-        Qn = Q[:nqc].numpy()
+        nqb = min(nq, a.cpu_queries)
+        Qn = Q[:nqb].numpy()
         t0 = time.perf_counter()
         skeys, sids = O.build_index(P, Xn, cfg["bs"])
         t_build = time.perf_counter() - t0
@@ -179,17 +208,17 @@ def main():
         ref = O.query(skeys, sids, Xn, Qn, qproj, M, L, cfg["bs"], cfg["ts"], k, cfg["outer"])
         t_query = time.perf_counter() - t0
         agree = float(np.mean([len(set(x.tolist()) & set(y.tolist())) / k
-                               for x, y in zip(ids[:nqc].cpu().numpy(), ref["ids"])]))
+                               for x, y in zip(ids[:nqb].cpu().numpy(), ref["ids"])]))
         t0 = time.perf_counter()
-        Xt, Qt = torch.from_numpy(Xn), torch.from_numpy(Qn[:min(nqc, 128)])
+        Xt, Qt = torch.from_numpy(Xn), torch.from_numpy(Qn[:min(nqb, 128)])
         torch.cdist(Qt, Xt).topk(k, largest=False)
         t_exact = time.perf_counter() - t0
-        cpu = dict(value=nqc / t_query, unit="queries/s", cores=O.max_threads(), kind="port",
+        cpu = dict(value=nqb / t_query, unit="queries/s", cores=O.max_threads(), kind="port",
                    sample="oracle (CPU restatement of the reference algorithm) on the first %d "
                           "queries of the same workload, same (bs, ts, outer); build timed on "
-                          "all %d points" % (nqc, N),
+                          "all %d points" % (nqb, N),
                    build_points_per_s=N / t_build, set_agreement_with_gpu=agree,
-                   exact_cdist_topk_queries_per_s=min(nqc, 128) / t_exact,
+                   exact_cdist_topk_queries_per_s=min(nqb, 128) / t_exact,
                    host_cpus=os.cpu_count(), torch_threads=torch.get_num_threads())
 
     out = {
@@ -205,7 +234,9 @@ def main():
         "recall_at_k": recall, "recall_ok": recall >= 0.95,
         "build_points_per_s": N / build_wall,
         "per_query": {"visited": V, "candidates": C, "probes": S, "outer_steps": steps_q,
-                      "algorithmic_bytes": bytes_per_query},
+                      "algorithmic_bytes": bytes_per_query, "counter_sample_queries": nqc,
+                      "entries_streamed_by_timed_kernel": float(own[0]),
+                      "key_reads_by_timed_kernel": float(own[2])},
         "kernel_ms": {"traverse": trav_avg_ms, "merge": float(np.mean(merge_ms)),
                       "query_project": float(np.mean(qproj_ms))},
         "build": build,

@@ -208,9 +208,12 @@ void dci_oracle_normalize(float* P, int I, int dim) {
 }
 
 /* src/util_kernel.cu:45-80 with the call at src/dci_cuda_kernel.cu:167-169:
- * row-major out[R][C] = A[R][dim] . B[C][dim]^T, fp32 (sequential sum here;
- * cuBLAS's order is unspecified).  Build: A = directions, B = data -> [I][N].
- * Query (:802-803): A = queries, B = directions -> [nq][I]. */
+ * row-major out[R][C] = A[R][dim] . B[C][dim]^T in fp32.  cuBLAS's summation
+ * order is unspecified; this restatement fixes it as ONE fused multiply-add
+ * chain over k = 0..dim-1 starting from +0 (what a compiled CUDA loop with the
+ * default -fmad=true does), which any IEEE-754 machine reproduces bit for bit.
+ * Build: A = directions, B = data -> [I][N].  Query (:802-803): A = queries,
+ * B = directions -> [nq][I]. */
 void dci_oracle_matmul_nt(const float* A, const float* B, float* out, int64_t R,
                           int64_t C, int dim) {
 #pragma omp parallel for schedule(static)
@@ -219,8 +222,8 @@ void dci_oracle_matmul_nt(const float* A, const float* B, float* out, int64_t R,
             float acc = 0.0f;
             const float* a = A + r * dim;
             const float* b = B + c * dim;
-            for (int k = 0; k < dim; k++) acc += a[k] * b[k];
-            out[r * C + c] = acc;
+            for (int k = 0; k < dim; k++) acc = std::fmaf(a[k], b[k], acc);
+            out[r * C + c] = acc + 0.0f;   /* -0 -> +0, so equal keys always tie on the id */
         }
     }
 }
