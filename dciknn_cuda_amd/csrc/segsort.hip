@@ -89,6 +89,180 @@ __global__ void segsort_tile_kernel(const float* __restrict__ keys, SegGeom g,
     }
 }
 
+// ---------------------------------------------------------------------------
+// LDS radix sort of one whole slice (4096 < points <= 32256) by one workgroup
+// (1024 threads up to 15360 points, 512 threads with more items each above:
+// the register file, not LDS, limits items per thread): least-significant-digit passes of 4 bits over the order-preserving
+// 32-bit image of the key.  Every thread owns IPT consecutive items in
+// registers (key + packed id/rank); a pass counts digits in per-thread private
+// 16-bit LDS counters laid out digit-major, scans the 16384 counters, and moves
+// keys, then ids, through one LDS staging buffer.  Thread-private counters plus
+// the digit-major scan make every pass stable, so equal keys keep ascending ids.
+// Nibbles that are constant over the slice (typically the exponent's) are
+// skipped.  Global traffic: keys read once, sorted keys / ids / inverse written
+// once, all coalesced.
+constexpr int kRadixMax = 63 * 512;
+constexpr int kRadixMin = 4096;       // up to this the bitonic tile kernel is faster
+
+template <int kRadixThreads, int IPT>
+__global__ __launch_bounds__(kRadixThreads) void segsort_radix_kernel(
+    const float* __restrict__ keys, SegGeom g, float* __restrict__ skeys,
+    int32_t* __restrict__ sids, uint32_t* __restrict__ inv, uint16_t* __restrict__ lids) {
+    extern __shared__ uint32_t rs[];
+    uint32_t* stage = rs;                                         // IPT*1024 words
+    uint16_t* stage16 = reinterpret_cast<uint16_t*>(rs);
+    uint16_t* cnt = reinterpret_cast<uint16_t*>(rs + IPT * kRadixThreads);   // [16][threads]
+    uint32_t* cnt32 = rs + IPT * kRadixThreads;
+    uint32_t* misc = rs + IPT * kRadixThreads + 8 * kRadixThreads;   // 64 words
+
+    const int tid = threadIdx.x;
+    const int lane = tid & 63, wave = tid >> 6;
+    const int b = (int)(blockIdx.x % g.B);
+    const int64_t i = blockIdx.x / g.B;
+    const int64_t off = (int64_t)b * g.ppb;
+    const int n = (int)min(g.n - off, g.ppb);
+    if (n <= 0) return;
+    const int64_t base = i * g.n + off;
+
+    if (tid < 2) misc[32 + tid] = tid ? 0xffffffffu : 0u;        // OR / AND of all keys
+    for (int j = tid; j < IPT * kRadixThreads; j += kRadixThreads)
+        stage[j] = j < n ? f2ord(keys[base + j] + 0.0f) : 0xffffffffu;   // pads sort last and stay last
+    __syncthreads();
+    uint32_t k[IPT], rp[IPT];      // rp: id in the low half, rank / position in the high half
+    uint32_t vor = 0, vand = 0xffffffffu;
+#pragma unroll
+    for (int r = 0; r < IPT; r++) {
+        k[r] = stage[tid * IPT + r];
+        rp[r] = (uint32_t)(tid * IPT + r);
+        const bool real = tid * IPT + r < n;
+        vor |= real ? k[r] : 0u;
+        vand &= real ? k[r] : 0xffffffffu;
+    }
+    for (int o = 32; o > 0; o >>= 1) {
+        vor |= (uint32_t)__shfl_xor((int)vor, o, 64);
+        vand &= (uint32_t)__shfl_xor((int)vand, o, 64);
+    }
+    if (lane == 0) { atomicOr(&misc[32], vor); atomicAnd(&misc[33], vand); }
+    __syncthreads();
+    const uint32_t varying = misc[32] ^ misc[33];
+
+    for (int shift = 0; shift < 32; shift += 4) {
+        if (((varying >> shift) & 15u) == 0u) continue;          // same nibble everywhere
+        __syncthreads();
+        {   // count digits in thread-private LDS counters (no atomics, order-preserving)
+#pragma unroll
+            for (int w = 0; w < 8; w++) cnt32[tid + w * kRadixThreads] = 0;
+            __syncthreads();
+#pragma unroll
+            for (int r = 0; r < IPT; r++) {
+                const uint32_t a = ((k[r] >> shift) & 15u) * kRadixThreads + tid;
+                const uint32_t c = cnt[a];
+                cnt[a] = (uint16_t)(c + 1);
+                rp[r] = (rp[r] & 0xffffu) | (c << 16);
+            }
+        }
+        __syncthreads();
+        {   // exclusive scan of the 16*threads counters in memory order (digit-major)
+            uint32_t v[8];
+            uint32_t sum = 0;
+#pragma unroll
+            for (int w = 0; w < 8; w++) { v[w] = cnt32[tid * 8 + w]; sum += (v[w] & 0xffffu) + (v[w] >> 16); }
+            uint32_t incl = sum;
+#pragma unroll
+            for (int o = 1; o < 64; o <<= 1) {
+                const uint32_t t = (uint32_t)__shfl_up((int)incl, o, 64);
+                if (lane >= o) incl += t;
+            }
+            if (lane == 63) misc[wave] = incl;
+            __syncthreads();
+            uint32_t run = incl - sum;
+            for (int w2 = 0; w2 < wave; w2++) run += misc[w2];
+#pragma unroll
+            for (int w = 0; w < 8; w++) {
+                const uint32_t lo = v[w] & 0xffffu, hi = v[w] >> 16;
+                cnt32[tid * 8 + w] = run | ((run + lo) << 16);
+                run += lo + hi;
+            }
+        }
+        __syncthreads();
+        // an opaque copy of the shift keeps the compiler from holding all IPT counter
+        // addresses of the counting loop alive across the scan
+        int shift2 = shift;
+        asm volatile("" : "+s"(shift2));
+#pragma unroll
+        for (int r = 0; r < IPT; r++) {      // all counter reads first, then all stores:
+            const uint32_t a = ((k[r] >> shift2) & 15u) * kRadixThreads + tid;   // interleaved they
+            rp[r] += (uint32_t)cnt[a] << 16;                                      // would wait on each other
+            if ((r & 7) == 7) __builtin_amdgcn_sched_barrier(0);
+        }
+        // (scheduling fences every 8 items keep the unrolled loops from computing all
+        //  IPT addresses up front, which would spill registers)
+#pragma unroll
+        for (int r = 0; r < IPT; r++) {
+            stage[rp[r] >> 16] = k[r];
+            if ((r & 7) == 7) __builtin_amdgcn_sched_barrier(0);
+        }
+        __syncthreads();
+#pragma unroll
+        for (int r = 0; r < IPT; r++) {
+            k[r] = stage[tid * IPT + r];
+            if ((r & 7) == 7) __builtin_amdgcn_sched_barrier(0);
+        }
+        __syncthreads();
+#pragma unroll
+        for (int r = 0; r < IPT; r++) {
+            stage16[rp[r] >> 16] = (uint16_t)rp[r];
+            if ((r & 7) == 7) __builtin_amdgcn_sched_barrier(0);
+        }
+        __syncthreads();
+#pragma unroll
+        for (int r = 0; r < IPT; r++) {
+            rp[r] = stage16[tid * IPT + r];
+            if ((r & 7) == 7) __builtin_amdgcn_sched_barrier(0);
+        }
+    }
+
+    // results, through LDS so that every global write is coalesced
+    __syncthreads();
+#pragma unroll
+    for (int r = 0; r < IPT; r++) stage[tid * IPT + r] = k[r];
+    __syncthreads();
+    for (int j = tid; j < n; j += kRadixThreads) skeys[base + j] = ord2f(stage[j]);
+    __syncthreads();
+    uint16_t* pos_of = stage16 + IPT * kRadixThreads;            // second half of the staging buffer
+#pragma unroll
+    for (int r = 0; r < IPT; r++) {
+        const int pos = tid * IPT + r;
+        const uint32_t id = rp[r] & 0xffffu;
+        stage16[pos] = (uint16_t)id;
+        if (pos < n) pos_of[id] = (uint16_t)pos;                 // the first n sorted items are the real ones
+    }
+    __syncthreads();
+    for (int j = tid; j < n; j += kRadixThreads) {
+        const uint32_t id = stage16[j];
+        sids[base + j] = (int32_t)(off + id);
+        if (lids) lids[base + j] = (uint16_t)id;
+        if (inv) inv[base + j] = pos_of[j];
+    }
+}
+
+template <int NT, int IPT>
+static int launch_radix(const float* d_keys, const SegGeom& g, int num_indices, float* d_skeys,
+                        int32_t* d_sids, uint32_t* d_inv, uint16_t* d_lids, hipStream_t s) {
+    const size_t lds = (size_t)(IPT * NT + 8 * NT + 64) * sizeof(uint32_t);
+    static bool attr_done = false;
+    if (!attr_done) {
+        DCIH_HIP(hipFuncSetAttribute((const void*)segsort_radix_kernel<NT, IPT>,
+                                     hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds));
+        attr_done = true;
+    }
+    const int64_t blocks = (int64_t)num_indices * g.B;
+    hipLaunchKernelGGL((segsort_radix_kernel<NT, IPT>), dim3((unsigned)blocks), dim3(NT), lds, s,
+                       d_keys, g, d_skeys, d_sids, d_inv, d_lids);
+    DCIH_HIP(hipGetLastError());
+    return 0;
+}
+
 // One merge pass: within every slice, neighbouring sorted runs of length `run`
 // are merged into runs of 2*run.  A workgroup produces kMergeChunk outputs.
 __global__ __launch_bounds__(kMergeThreads) void segsort_merge_kernel(
@@ -149,7 +323,7 @@ __global__ void segsort_unpack_kernel(const unsigned long long* __restrict__ pac
 
 size_t segsort_tmp_bytes(int num_indices, int64_t n, int block_size) {
     const int64_t ppb = (n + block_size - 1) / block_size;
-    if (ppb <= kTileCap) return 0;
+    if (ppb <= 63 * 512) return 0;       // one LDS pass (bitonic tile or radix kernel)
     return (size_t)2 * num_indices * n * sizeof(unsigned long long);
 }
 
@@ -186,6 +360,15 @@ int segsort(const float* d_keys, int num_indices, int64_t n, int block_size,
         attr_done[0] = true;
     }
 
+    if (g.ppb > kRadixMin && g.ppb <= kRadixMax) {
+        // odd items-per-thread keep the blocked LDS accesses free of bank conflicts
+#define DCIH_RADIX(NT, IPT) \
+    if (g.ppb <= (int64_t)(NT) * (IPT))  \
+        return launch_radix<NT, IPT>(d_keys, g, num_indices, d_skeys, d_sids, d_inv, d_lids, s)
+        DCIH_RADIX(1024, 3); DCIH_RADIX(1024, 7); DCIH_RADIX(1024, 11); DCIH_RADIX(1024, 15);
+        DCIH_RADIX(512, 37); DCIH_RADIX(512, 45); DCIH_RADIX(512, 53); DCIH_RADIX(512, 63);
+#undef DCIH_RADIX
+    }
     if (g.tiles == 1) {
         hipLaunchKernelGGL(segsort_tile_kernel<true>, dim3((unsigned)blocks), dim3(threads), lds, s,
                            d_keys, g, d_skeys, d_sids, d_inv, d_lids, (unsigned long long*)nullptr, np2);

@@ -99,7 +99,9 @@ def test_project_same_vector_same_bits(gpu):
 # ------------------------------------------------------------ segmented sort
 @pytest.mark.parametrize("n,I,B", [(3000, 20, 100), (1000, 3, 7), (10, 2, 16), (1, 1, 1),
                                    (16384, 2, 1), (16385, 2, 1), (50000, 3, 1), (100000, 2, 3),
-                                   (4099, 5, 4)])
+                                   (4099, 5, 4), (2049, 2, 1), (4096, 2, 1), (4097, 2, 1), (8200, 3, 2), (10000, 3, 1), (15360, 2, 1), (15361, 2, 1),
+                                   (25000, 2, 2), (62500, 3, 2), (32256, 1, 1), (32257, 1, 1),
+                                   (70000, 2, 3)])
 def test_segsort_matches_oracle(gpu, oracle, n, I, B):
     rng = np.random.default_rng(n * 31 + B)
     keys = rng.standard_normal((I, n)).astype(np.float32)
@@ -108,6 +110,23 @@ def test_segsort_matches_oracle(gpu, oracle, n, I, B):
     rk, ri = oracle.segsort(keys, B)
     np.testing.assert_array_equal(sk, rk)
     np.testing.assert_array_equal(si, ri)
+
+
+def test_index_arrays_are_consistent(gpu):
+    """sids, the 16-bit partition-relative ids and the inverse permutation describe
+    one and the same order (checked through a query that uses all three)."""
+    rng = np.random.default_rng(3)
+    for n, B in [(40_000, 2), (9_000, 3), (1_000, 5)]:
+        X = rng.standard_normal((n, 8)).astype(np.float32)
+        dci = gpu.DCI(8, 2, 3, B, 4, seed=3)
+        dci.add(torch.from_numpy(X).cuda())
+        sk, si = engine_index(dci)
+        ppb = -(-n // B)
+        for b in range(B):
+            lo, hi = b * ppb, min(n, (b + 1) * ppb)
+            assert np.all(np.diff(sk[:, lo:hi], axis=1) >= 0)
+            assert np.array_equal(np.sort(si[:, lo:hi], axis=1), np.tile(np.arange(lo, hi), (6, 1)))
+        dci.free()
 
 
 def test_segsort_invariants_large(gpu):
