@@ -55,9 +55,10 @@ struct BlockLayout {
     int off_chunk0;   // per stream: global index of its first 16-byte chunk (2I 64-bit words)
     int off_comp;     // per composite: rho bits, K, active, previous K (4 * M words)
     int off_q;        // query row
+    int off_samp;     // per stream: 16 sampled window priorities of the current epoch's range
     int off_promo, off_events, off_acc, off_sort, off_cnt;
     int event_cap;    // promotions waiting for the other composites (= accepted candidates per replay)
-    int sort_cap;     // power of two >= kcap + event_cap: top-k plus one batch of candidates
+    int sort_cap;     // power of two >= kcap + 128: top-k plus one batch of candidates
     size_t lds_bytes;
 };
 
@@ -83,8 +84,9 @@ BlockLayout make_block_layout(const QueryArgs& a) {
     // small tables keep more workgroups resident per CU; an item that overflows them
     // is redone by the step-by-step kernel
     y.event_cap = 512;
-    y.sort_cap = 2;
-    while (y.sort_cap < a.kcap + y.event_cap) y.sort_cap <<= 1;
+    y.sort_cap = 256;          // top-k plus a batch of at least 128 new candidates
+    while (y.sort_cap < a.kcap + 128) y.sort_cap <<= 1;
+    y.off_samp = o;     o += 2 * I * 16 * 4;
     y.off_promo = o;    o += kPromoCap * 4;
     y.off_acc = o;      o += y.event_cap * 4;
     o = (o + 15) & ~15;
@@ -170,6 +172,7 @@ __global__ __launch_bounds__(NT) void traverse_block_kernel(QueryArgs a, BlockLa
     uint32_t* s_active = s_K + a.M;
     uint32_t* s_Kprev = s_active + a.M;
     float* s_q = reinterpret_cast<float*>(smem + y.off_q);
+    uint32_t* s_samp = reinterpret_cast<uint32_t*>(smem + y.off_samp);
     uint32_t* promo = reinterpret_cast<uint32_t*>(smem + y.off_promo);
     uint32_t* acc = reinterpret_cast<uint32_t*>(smem + y.off_acc);
     unsigned long long* events = reinterpret_cast<unsigned long long*>(smem + y.off_events);
@@ -255,6 +258,26 @@ __global__ __launch_bounds__(NT) void traverse_block_kernel(QueryArgs a, BlockLa
         st.n = n; st.T = T; st.p = s_p[i]; st.side = s & 1; st.q = s_qp[i];
         return st;
     };
+    // count_below over the epoch's range [cprev, c) of stream sidx, narrowed first by
+    // the 15 priorities sampled from that range (LDS), then by key reads
+    auto count_in_epoch = [&](int sidx, uint32_t x, bool strict) {
+        int lo = s_cprev[sidx], hi = s_c[sidx];
+        const int len = hi - lo;
+        if (len >= 32) {
+            const uint32_t* tab = s_samp + sidx * 16;
+            int tl = 0, th = 15;            // number of samples t in 1..15 below x (monotone)
+            while (tl < th) {
+                const int mid = (tl + th + 1) >> 1;
+                const uint32_t v = tab[mid];
+                if (strict ? v < x : v <= x) tl = mid; else th = mid - 1;
+            }
+            const int base0 = lo;
+            if (tl > 0) lo = base0 + (int)(((int64_t)len * tl) >> 4) + 1;
+            if (tl < 15) hi = base0 + (int)(((int64_t)len * (tl + 1)) >> 4);
+        }
+        return count_below(load_stream(sidx), x, strict, lo, hi, probes);
+    };
+
     // Adds (or, for undo, removes) the visits of windows [cprev, c) of all streams.
     // The loop is bound by vector-ALU issue (about 8 instructions and one LDS
     // atomic per visit), so it reads partition-relative 16-bit ids, eight per
@@ -466,6 +489,17 @@ __global__ __launch_bounds__(NT) void traverse_block_kernel(QueryArgs a, BlockLa
         }
 
         // ---- 4. exact step of every promotion -----------------------------------
+        if (np > 0) {     // sample every stream's new range once; all rankings of the epoch share it
+            for (int idx = tid; idx < S * 15; idx += NT) {
+                const int sidx = idx / 15, t = idx - sidx * 15 + 1;
+                const int lo = s_cprev[sidx], len = s_c[sidx] - lo;
+                if (len >= 32) {
+                    probes++;
+                    s_samp[sidx * 16 + t] = stream_prio_bits(load_stream(sidx), lo + (int)(((int64_t)len * t) >> 4));
+                }
+            }
+            __syncthreads();
+        }
         {
             constexpr int kGroup = 32;
             const int gl = tid & (kGroup - 1);
@@ -510,15 +544,14 @@ __global__ __launch_bounds__(NT) void traverse_block_kernel(QueryArgs a, BlockLa
                 for (int s2 = gl; s2 < 2 * a.L; s2 += kGroup) {
                     const int h2 = s2 >> 1, side2 = s2 & 1;
                     const int sidx = 2 * (m * a.L + h2) + side2;
-                    const int lo = s_cprev[sidx], hi = s_c[sidx];
                     int c;
                     if (h2 == w_h) {
                         const bool corner = s_p[m * a.L + h2] == n - 1 && T >= 2;  // ghost window first
                         if (side2 == w_side) c = w_j;
                         else if (corner) c = w_side ? 0 : s_ns[sidx];
-                        else c = count_below(load_stream(sidx), w_bits, w_side == 0, lo, hi, probes);
+                        else c = count_in_epoch(sidx, w_bits, w_side == 0);
                     } else {
-                        c = count_below(load_stream(sidx), w_bits, h2 > w_h, lo, hi, probes);
+                        c = count_in_epoch(sidx, w_bits, h2 > w_h);
                     }
                     rank += (uint32_t)c;
                 }
@@ -609,10 +642,11 @@ __global__ __launch_bounds__(NT) void traverse_block_kernel(QueryArgs a, BlockLa
         // ---- 6. distances of the accepted candidates, merged into the top-k ---------
         const int nacc = (int)misc[kAccCount];
         const bool stop = misc[kStop] != 0;
-        if (nacc > 0) {
+        for (int done = 0; done < nacc;) {      // in batches that fit beside the top-k
             const int topn = (int)misc[kTopN];
-            for (int c = wave; c < nacc; c += kWaves) {
-                const int64_t pt = off + acc[c];
+            const int batch = min(nacc - done, y.sort_cap - topn);
+            for (int c = wave; c < batch; c += kWaves) {
+                const int64_t pt = off + acc[done + c];
                 const float* row = a.data + pt * a.dim;
                 float sum = 0.f;
                 for (int j = lane; j < a.dim; j += kWave) {
@@ -624,13 +658,15 @@ __global__ __launch_bounds__(NT) void traverse_block_kernel(QueryArgs a, BlockLa
                     sortbuf[topn + c] = ((unsigned long long)__builtin_bit_cast(uint32_t, dist) << 32) | (uint32_t)pt;
             }
             int np2 = 2;
-            while (np2 < topn + nacc) np2 <<= 1;
-            for (int j = topn + nacc + tid; j < np2; j += NT) sortbuf[j] = ~0ull;
+            while (np2 < topn + batch) np2 <<= 1;
+            for (int j = topn + batch + tid; j < np2; j += NT) sortbuf[j] = ~0ull;
             bitonic_sort_u64(sortbuf, np2);
-            if (tid == 0) {
-                misc[kTopN] = (uint32_t)min(a.kcap, topn + nacc);
-                misc[kAccCount] = 0;
-            }
+            if (tid == 0) misc[kTopN] = (uint32_t)min(a.kcap, topn + batch);
+            done += batch;
+            __syncthreads();
+        }
+        if (nacc > 0) {
+            if (tid == 0) misc[kAccCount] = 0;
             __syncthreads();
         }
         phase(7);
@@ -642,9 +678,18 @@ __global__ __launch_bounds__(NT) void traverse_block_kernel(QueryArgs a, BlockLa
             uint32_t kmax = 0, dk_lead = 1;
             for (int m = 0; m < a.M; m++)
                 if (s_K[m] >= kmax) { kmax = s_K[m]; dk_lead = max(1u, s_K[m] - s_Kprev[m]); }
-            float k_target = (float)kmax + (shrunk ? 1.0f : 2.0f) * (float)dk_lead;
-            if (hint > 0.0f && !shrunk)
+            // where to land next (steps per composite): just past the stop step once
+            // c0 >= k; else by the hint; else twice the last stride
+            float k_target = (float)kmax + 2.0f * (float)dk_lead;
+            const float need = (float)(a.stop_at > 0 ? a.stop_at : 1);
+            if (misc[kArmed]) {
+                const float t_armed = (float)(((unsigned long long)misc[kArmedHi] << 32) | misc[kArmedLo]);
+                k_target = fmaxf(t_armed + 1.0f, need) + (float)S;
+            } else if (hint > 0.0f) {
                 k_target = (float)kmax < 0.7f * hint ? 0.75f * hint : 1.12f * (float)kmax + (float)S;
+            }
+            k_target = fminf(k_target, 2.0f * (float)kmax + 16.0f * (float)S);
+            if (shrunk) k_target = fminf(k_target, (float)kmax + (float)dk_lead);
             __syncthreads();
             if (tid < S) {
                 const int m = (tid >> 1) / a.L;
