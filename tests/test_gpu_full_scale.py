@@ -1,0 +1,84 @@
+"""Full-size checks on workload C2 (1M x 128, m=2, L=10, k=10): the sizes are far
+beyond what the CPU oracle covers in seconds for all queries, so the checks are
+size-independent properties plus the oracle on a small query sample."""
+import numpy as np
+import pytest
+import torch
+
+from util import set_agreement
+
+pytestmark = pytest.mark.gpu
+
+B, T, OUTER, K = 32, 4, 500, 10
+
+
+@pytest.fixture(scope="module")
+def c2(gpu):
+    from dciknn_cuda_amd import workloads
+    X, Q = workloads.c2()
+    Xd, Qd = X.cuda(), Q[:2048].contiguous().cuda()
+    dci = gpu.DCI(128, 2, 10, B, T, seed=4)
+    dci.add(Xd)
+    yield dict(X=X, Q=Q[:2048], Xd=Xd, Qd=Qd, dci=dci)
+    dci.free()
+
+
+def test_recall_and_self_consistency(c2):
+    dci, Xd, Qd = c2["dci"], c2["Xd"], c2["Qd"]
+    ids, dists = dci.query(Qd, K, OUTER, return_int=True)
+    xn = (Xd * Xd).sum(1)
+    gt = torch.cat([(xn[None] - 2 * Qd[s:s + 512] @ Xd.T).topk(K, largest=False).indices
+                    for s in range(0, Qd.shape[0], 512)])
+    recall = (ids.long()[:, :, None] == gt[:, None, :]).any(2).float().mean().item()
+    assert recall >= 0.95, recall
+    assert torch.all(dists[:, 1:] >= dists[:, :-1])
+    assert torch.all(ids >= 0) and torch.all(ids < Xd.shape[0])
+    # a returned distance is the exact distance of the returned id
+    d = (Xd[ids.long()] - Qd[:, None, :]).norm(dim=2)
+    assert torch.allclose(d, dists, rtol=1e-5, atol=1e-4)
+    # no id twice in a row of results
+    s = ids.sort(dim=1).values
+    assert torch.all(s[:, 1:] != s[:, :-1])
+
+
+def test_batch_and_step_kernels_agree(c2):
+    dci, Qd = c2["dci"], c2["Qd"][:192].contiguous()
+    dci.set_traversal("batch")
+    ib, db, cb = dci.query(Qd, K, OUTER, return_int=True, return_counters=True)
+    dci.set_traversal("step")
+    i_s, d_s, cs = dci.query(Qd, K, OUTER, return_int=True, return_counters=True)
+    dci.set_traversal("auto")
+    assert torch.equal(db, d_s)
+    assert torch.equal(ib, i_s)
+    assert torch.equal(cb[:, 1], cs[:, 1]) and torch.equal(cb[:, 3], cs[:, 3])   # candidates, steps
+    assert torch.all(cb[:, 0] >= cs[:, 0])                                        # streamed >= visited
+
+
+def test_oracle_end_to_end_on_a_sample(c2, oracle):
+    """Only data, queries and directions are shared with the oracle."""
+    dci = c2["dci"]
+    nq = 48
+    ids, dists = dci.query(c2["Qd"][:nq].contiguous(), K, OUTER, return_int=True)
+    ref = oracle.knn(dci.directions.numpy(), c2["X"].numpy(), c2["Q"][:nq].numpy(), 2, 10, B, T, K, OUTER)
+    assert set_agreement(ids.cpu().numpy(), ref["ids"]) >= 0.999
+    np.testing.assert_allclose(dists.cpu().numpy(), ref["dists"], rtol=1e-5)
+
+
+def test_results_do_not_depend_on_batching_or_history(c2):
+    """Same answers for a query alone, in a batch, and after the epoch-size hints warmed up."""
+    dci, Qd = c2["dci"], c2["Qd"]
+    a = dci.query(Qd[:256].contiguous(), K, OUTER, return_int=True)
+    b = dci.query(Qd[100:101].contiguous(), K, OUTER, return_int=True)
+    c = dci.query(Qd[:256].contiguous(), K, OUTER, return_int=True)
+    assert torch.equal(a[0][100], b[0][0]) and torch.equal(a[1][100], b[1][0])
+    assert torch.equal(a[0], c[0]) and torch.equal(a[1], c[1])
+
+
+def test_more_iterations_never_worse(c2):
+    dci, Qd = c2["dci"], c2["Qd"][:128].contiguous()
+    prev = None
+    for outer in (100, 20000, 60000, 200000):
+        _, d = dci.query(Qd, K, outer)
+        if prev is not None:
+            assert torch.all(d <= prev * (1 + 1e-6))
+        prev = d

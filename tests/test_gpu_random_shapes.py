@@ -1,0 +1,82 @@
+"""Randomised traversal parity: both query kernels against the CPU oracle on many
+small seeded shapes, including the awkward corners (L = 1, where every visit is a
+promotion; duplicated points, where priorities tie everywhere; windows wider
+than a partition; budgets of 0 and 1 iterations; tiny max_num_candidates)."""
+import numpy as np
+import pytest
+import torch
+
+from util import engine_index, engine_project, set_agreement
+
+pytestmark = pytest.mark.gpu
+
+
+def _shape(rng):
+    M = int(rng.integers(1, 4))
+    L = int(rng.choice([1, 2, 3, 5, 8, 15, 16, 20]))
+    while M * L > 64:
+        L //= 2
+    n = int(rng.choice([1, 2, 7, 50, 333, 1500, 6000]))
+    B = int(rng.choice([1, 2, 3, 9, 40]))
+    T = int(rng.choice([1, 2, 3, 8, 17, 64, 130]))
+    k = int(min(n, rng.choice([1, 3, 10, 40])))
+    outer = int(rng.choice([0, 1, 2, 7, 40, 100000]))
+    max_cand = int(rng.choice([1, k, 10 * k, 10 ** 6]))
+    dim = int(rng.choice([1, 2, 5, 16, 33]))
+    kind = str(rng.choice(["normal", "dup", "grid", "far"]))
+    return M, L, n, B, T, k, outer, max_cand, dim, kind
+
+
+def _points(rng, n, nq, dim, kind):
+    if kind == "dup":       # every point appears several times
+        base = rng.standard_normal((max(1, n // 4), dim))
+        x = base[rng.integers(0, base.shape[0], n)]
+        q = base[rng.integers(0, base.shape[0], nq)] + 0.01 * rng.standard_normal((nq, dim))
+    elif kind == "grid":
+        x = rng.integers(0, 4, (n, dim)).astype(float)
+        q = rng.integers(0, 4, (nq, dim)).astype(float)
+    elif kind == "far":     # queries outside the data on every direction
+        x = rng.standard_normal((n, dim))
+        q = 50.0 + rng.standard_normal((nq, dim))
+    else:
+        x = rng.standard_normal((n, dim))
+        q = rng.standard_normal((nq, dim))
+    return x.astype(np.float32), q.astype(np.float32)
+
+
+@pytest.mark.parametrize("seed", range(150))
+def test_random_shape(gpu, oracle, seed):
+    from dciknn_cuda_amd import _capi
+    rng = np.random.default_rng(1000 + seed)
+    M, L, n, B, T, k, outer, max_cand, dim, kind = _shape(rng)
+    nq = 6
+    X, Q = _points(rng, n, nq, dim, kind)
+    xd, qd = torch.from_numpy(X).cuda(), torch.from_numpy(Q).cuda()
+    ref = None
+    for traversal in ("step", "auto"):
+        dci = gpu.DCI(dim, M, L, B, T, seed=seed, traversal=traversal)
+        dci.add(xd)
+        ids = torch.empty((nq, k), dtype=torch.int32, device="cuda")
+        dists = torch.empty((nq, k), dtype=torch.float32, device="cuda")
+        ctr = torch.empty((nq, 4), dtype=torch.int64, device="cuda")
+        _capi.check(dci._lib.dcih_query(dci._dci_inst, dim, nq, qd.data_ptr(), k, 0, outer, max_cand,
+                                        B, T, ids.data_ptr(), dists.data_ptr(), ctr.data_ptr(),
+                                        torch.cuda.current_stream().cuda_stream))
+        torch.cuda.synchronize()
+        if ref is None:
+            skeys, sids = engine_index(dci)
+            qproj = engine_project(dci.directions.numpy(), Q).T.copy()
+            ref = oracle.query(skeys, sids, X, Q, qproj, M, L, B, T, k, outer, max_cand=max_cand)
+        dci.free()
+        tag = "%s %s" % (traversal, (M, L, n, B, T, k, outer, max_cand, dim, kind))
+        ids, dists, ctr = ids.cpu().numpy(), dists.cpu().numpy(), ctr.cpu().numpy()
+        rc = ref["counters"].astype(np.int64)
+        np.testing.assert_array_equal(ctr[:, 1], rc[:, 1], err_msg="candidates " + tag)
+        np.testing.assert_array_equal(ctr[:, 3], rc[:, 3], err_msg="steps " + tag)
+        if traversal == "step":
+            np.testing.assert_array_equal(ctr[:, 0], rc[:, 0], err_msg="visits " + tag)
+        np.testing.assert_allclose(dists, ref["dists"], rtol=1e-5, atol=1e-6, err_msg=tag)
+        if kind == "normal" or kind == "far":     # no exact distance ties: ids must agree
+            assert set_agreement(ids, ref["ids"]) == 1.0, tag
+        else:                                     # ties: same (id present / absent) pattern
+            np.testing.assert_array_equal(ids < 0, ref["ids"] < 0, err_msg=tag)
