@@ -47,5 +47,40 @@ def build_library(verbose=False):
     return LIB
 
 
+EXT = os.path.join(HERE, "_dci_cuda.so")
+
+
+def build_extension(verbose=False):
+    """Compile the torch C++ extension `_dci_cuda` (host side, g++) against libdci_hip.so."""
+    import sysconfig
+
+    import torch
+    from torch.utils import cpp_extension as ce
+    if not os.path.exists(LIB):
+        build_library(verbose)
+    tlib = os.path.join(os.path.dirname(torch.__file__), "lib")
+    cmd = [os.environ.get("CXX", "g++"), "-O2", "-std=c++17", "-fPIC", "-shared",
+           "-D__HIP_PLATFORM_AMD__=1", "-DUSE_ROCM=1", "-DTORCH_EXTENSION_NAME=_dci_cuda",
+           "-DTORCH_API_INCLUDE_EXTENSION_H", "-DPYBIND11_COMPILER_TYPE=\"_gcc\"",
+           "-DPYBIND11_STDLIB=\"_libstdcpp\"", "-DPYBIND11_BUILD_ABI=\"_cxxabi1011\"",
+           "-D_GLIBCXX_USE_CXX11_ABI=%d" % int(torch._C._GLIBCXX_USE_CXX11_ABI),
+           "-Wno-deprecated-declarations"]
+    for inc in ce.include_paths() + ["/opt/rocm/include", sysconfig.get_paths()["include"]]:
+        cmd += ["-isystem", inc]
+    cmd += [os.path.join(CSRC, "_dci_cuda.cpp"), "-o", EXT,
+            "-L" + tlib, "-L" + HERE, "-ldci_hip", "-lc10", "-lc10_hip", "-ltorch_cpu", "-ltorch_hip",
+            "-ltorch", "-ltorch_python", "-Wl,-rpath,$ORIGIN", "-Wl,-rpath," + tlib]
+    r = subprocess.run(cmd, capture_output=True, text=True)
+    if r.returncode != 0:
+        raise RuntimeError("building _dci_cuda failed:\n%s" % r.stderr[-4000:])
+    if verbose and r.stderr.strip():
+        print(r.stderr[-2000:], file=sys.stderr)
+    return EXT
+
+
+def build_all(verbose=False):
+    return build_library(verbose), build_extension(verbose)
+
+
 if __name__ == "__main__":
-    print(build_library(verbose=True))
+    print(build_all(verbose=True))

@@ -2,7 +2,10 @@
 
 `DCI` and `MDCI` keep the public behaviour of the reference's
 dciknn_cuda/core.py:25-169 (argument names, defaults, exception types, return
-shapes and dtypes) on top of libdci_hip.so.  Additions, all keyword-only and
+shapes and dtypes).  Like there, the seven `_dci_*` functions come from the
+compiled torch extension `_dci_cuda` (csrc/_dci_cuda.cpp), which calls the
+C-ABI of libdci_hip.so; what the reference has no function for (directions,
+counters, kernel choice) goes to the C-ABI directly.  Additions, all keyword-only and
 optional: `seed` / `directions` at construction and the `directions` property
 (the reference can neither seed, inject nor read its directions), and
 `return_int` / `return_counters` on `query`, and `traversal` / `set_traversal`
@@ -11,6 +14,7 @@ to pick the query kernel.
 import torch
 
 from . import _capi
+from . import _dci_cuda as _ext   # built by `python -m dciknn_cuda_amd.build`; no fallback
 
 
 def _stream_ptr(device):
@@ -29,11 +33,10 @@ class DCI(object):
         self._device = torch.device("cuda", device if isinstance(device, int) else
                                     torch.device(device).index or 0)
         self._lib = _capi.lib()
-        handle = _capi.ctypes.c_void_p()
-        _capi.check(self._lib.dcih_create(dim, num_comp_indices, num_simp_indices,
-                                          self._device.index, seed,
-                                          _capi.ctypes.byref(handle)))
-        self._dci_inst = handle
+        self._capsule = _ext._dci_new(dim, num_comp_indices, num_simp_indices,
+                                      self._device.index, seed)
+        # the same handle as a plain pointer, for direct C-ABI calls
+        self._dci_inst = _capi.ctypes.c_void_p(_ext._dci_handle(self._capsule))
         self._array = None
         self._block_size = bs
         self._thread_size = ts
@@ -115,9 +118,8 @@ class DCI(object):
         self._check_data(data)
         if data.device != self._device:
             raise ValueError("tensor is on %s but this DCI instance lives on %s" % (data.device, self._device))
-        _capi.check(self._lib.dcih_add(self._dci_inst, self._dim, data.shape[0], data.data_ptr(),
-                                       self._block_size, self._thread_size,
-                                       _stream_ptr(self._device)))
+        _ext._dci_add(self._capsule, self._dim, data.shape[0], data.flatten(),
+                      self._block_size, self._thread_size)
         self.num_points = data.shape[0]
         self._array = data   # the index borrows this memory
 
@@ -141,6 +143,13 @@ class DCI(object):
             raise ValueError("num_neighbours exceeds the number of indexed points")
         max_num_candidates = 10 * num_neighbours
         nq = _query.shape[0]
+        if not return_int and not return_counters:
+            # the reference's own route: one flat float tensor, ids first (core.py:90-92)
+            _query_result = _ext._dci_query(self._capsule, self._dim, nq, _query.flatten(),
+                                            num_neighbours, blind, num_outer_iterations,
+                                            max_num_candidates, self._block_size, self._thread_size)
+            half = _query_result.shape[0] // 2
+            return _query_result[:half].reshape(nq, -1), _query_result[half:].reshape(nq, -1)
         ids = torch.empty((nq, num_neighbours), dtype=torch.int32, device=self._device)
         dists = torch.empty((nq, num_neighbours), dtype=torch.float32, device=self._device)
         counters = None
@@ -160,19 +169,19 @@ class DCI(object):
 
     def clear(self):
         self._require_handle()
-        _capi.check(self._lib.dcih_clear(self._dci_inst))
+        _ext._dci_clear(self._capsule)
         self.num_points = 0
         self._array = None
 
     def reset(self):
         self._require_handle()
-        _capi.check(self._lib.dcih_reset(self._dci_inst))
+        _ext._dci_reset(self._capsule)
         self.num_points = 0
         self._array = None
 
     def free(self):
         if getattr(self, "_dci_inst", None) is not None:
-            self._lib.dcih_free(self._dci_inst)
+            _ext._dci_free(self._capsule)
             self._dci_inst = None
         self.num_points = 0
         self._array = None
@@ -206,7 +215,17 @@ class MDCI(object):
         else:
             _query = query
         _query = _query.detach().clone().to(self.dcis[0]._device)
-        nns, dists = self.dcis[0].query(_query, num_neighbours, num_outer_iterations, blind)
+        d0 = self.dcis[0]
+        d0._check_data(_query)
+        if blind:
+            raise NotImplementedError("blind querying is not available in this build")
+        max_num_candidates = 10 * num_neighbours
+        res = _ext._dci_multi_query([dc._capsule for dc in self.dcis], d0._dim, _query.shape[0],
+                                    [_query.flatten()], num_neighbours, blind, num_outer_iterations,
+                                    max_num_candidates, d0._block_size, d0._thread_size)
+        half = res[0].shape[0] // 2
+        nns = res[0][:half].reshape(_query.shape[0], -1)
+        dists = res[0][half:].reshape(_query.shape[0], -1)
         _, sort_indices = torch.sort(dists, dim=1, stable=True)
         sort_indices = sort_indices[:, :num_neighbours]
         return torch.gather(nns, 1, sort_indices), torch.gather(dists, 1, sort_indices)

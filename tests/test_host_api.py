@@ -46,6 +46,14 @@ def test_null_and_bad_arguments_return_status_codes():
         _capi.check(lib.dcih_clear(None))
 
 
+def test_extension_module_exports_the_reference_names():
+    """The seven functions dciknn_cuda/core.py:19 imports, plus the handle accessor."""
+    from dciknn_cuda_amd import _dci_cuda
+    for name in ("_dci_new", "_dci_add", "_dci_query", "_dci_clear", "_dci_reset", "_dci_free",
+                 "_dci_multi_query", "_dci_handle"):
+        assert callable(getattr(_dci_cuda, name))
+
+
 def test_constructor_needs_a_gpu():
     if torch.cuda.is_available():
         pytest.skip("a GPU is present")
@@ -59,7 +67,7 @@ def _bare(dim=4):
     from dciknn_cuda_amd import DCI
     d = DCI.__new__(DCI)
     d._dim, d._num_comp_indices, d._num_simp_indices = dim, 2, 3
-    d._dci_inst, d._array, d.num_points = None, None, 0
+    d._dci_inst, d._capsule, d._array, d.num_points = None, None, None, 0
     return d
 
 
