@@ -51,7 +51,7 @@ enum Misc {   // 32-bit scalars shared by the workgroup; kStreamedLo must stay 8
 struct BlockLayout {
     int cbits, wpc, seen_words, counter_words;
     int off_idx;      // per simple index: p, qp            (2 * I words)
-    int off_stream;   // per stream: consumed, previous, total, range lo/hi, chunks, pos0, prefix (9 * 2I + 1 words, incl. the stride)
+    int off_stream;   // per stream: consumed, previous, total, range lo/hi, chunks, pos0, prefix (10 * 2I + 1 words, incl. stride and composite number)
     int off_chunk0;   // per stream: global index of its first 16-byte chunk (2I 64-bit words)
     int off_comp;     // per composite: rho bits, K, active, previous K (4 * M words)
     int off_q;        // query row
@@ -76,7 +76,7 @@ BlockLayout make_block_layout(const QueryArgs& a) {
     y.counter_words = a.M * y.wpc + y.seen_words;
     int o = kMiscWords * 4;
     y.off_idx = o;      o += 2 * I * 4;
-    y.off_stream = o;   o += (9 * 2 * I + 2) * 4;
+    y.off_stream = o;   o += (10 * 2 * I + 2) * 4;
     o = (o + 7) & ~7;
     y.off_chunk0 = o;   o += 2 * I * 8;
     y.off_comp = o;     o += 4 * a.M * 4;
@@ -148,8 +148,10 @@ __device__ inline unsigned long long pack_event(uint32_t time, int m, bool lane0
            ((unsigned long long)(lane0 ? 1u : 0u) << 25) | local;
 }
 
-template <int NT, int CBITS>
-__global__ __launch_bounds__(NT) void traverse_block_kernel(QueryArgs a, BlockLayout y) {
+// MINW = waves per SIMD the register allocation must leave room for: LDS decides how
+// many workgroups fit a CU, and the kernel should not be the tighter limit.
+template <int NT, int CBITS, int MINW>
+__global__ __launch_bounds__(NT, MINW) void traverse_block_kernel(QueryArgs a, BlockLayout y) {
     constexpr uint32_t kFpw = 32 / CBITS;                       // counters per 32-bit word
     constexpr int kFshift = CBITS == 4 ? 3 : 2;                 // log2(kFpw)
     constexpr uint32_t kCmask = (1u << CBITS) - 1u;
@@ -165,7 +167,8 @@ __global__ __launch_bounds__(NT) void traverse_block_kernel(QueryArgs a, BlockLa
     int* s_nch = s_rb + 2 * a.M * a.L;                                // 16-byte chunks the range touches
     int* s_pos0 = s_nch + 2 * a.M * a.L;                              // position of the first chunk's first id
     int* s_stride = s_pos0 + 2 * a.M * a.L;                           // windows to try next epoch
-    int* s_pref = s_stride + 2 * a.M * a.L;                           // whole-chunk prefix sums (2I + 1)
+    int* s_mof = s_stride + 2 * a.M * a.L;                            // composite the stream belongs to
+    int* s_pref = s_mof + 2 * a.M * a.L;                              // whole-chunk prefix sums (2I + 1)
     long long* s_chunk0 = reinterpret_cast<long long*>(smem + y.off_chunk0);
     uint32_t* s_rho = reinterpret_cast<uint32_t*>(smem + y.off_comp); // per composite
     uint32_t* s_K = s_rho + a.M;
@@ -229,6 +232,7 @@ __global__ __launch_bounds__(NT) void traverse_block_kernel(QueryArgs a, BlockLa
         for (int side = 0; side < 2; side++) {
             s_ns[2 * tid + side] = stream_windows(n, T, p, side);
             s_c[2 * tid + side] = 0;
+            s_mof[2 * tid + side] = tid / a.L;
         }
     }
     __syncthreads();
@@ -347,24 +351,24 @@ __global__ __launch_bounds__(NT) void traverse_block_kernel(QueryArgs a, BlockLa
         // whole chunks
         const int total = s_pref[S];
         int cur = 0;
-        for (int g0 = 0; g0 < total; g0 += NT * kUnroll) {
-            uint4 r[kUnroll];
-            int sreg[kUnroll];
+        auto fetch = [&](int g0, uint4 (&r)[kUnroll], int (&mr)[kUnroll]) {
 #pragma unroll
             for (int u = 0; u < kUnroll; u++) {
                 const int g = g0 + u * NT + tid;
-                sreg[u] = -1;
+                mr[u] = -1;
                 if (g < total) {
                     while (g >= s_pref[cur + 1]) cur++;
-                    sreg[u] = cur;
+                    mr[u] = s_mof[cur];
                     r[u] = all[s_chunk0[cur] + 1 + (g - s_pref[cur])];
                 }
             }
+        };
+        auto process = [&](const uint4 (&r)[kUnroll], const int (&mr)[kUnroll]) {
             if (undo) {
 #pragma unroll
                 for (int u = 0; u < kUnroll; u++) {
-                    if (sreg[u] < 0) continue;
-                    uint32_t* mcnt = cnt + (size_t)((sreg[u] >> 1) / a.L) * y.wpc;
+                    if (mr[u] < 0) continue;
+                    uint32_t* mcnt = cnt + (size_t)mr[u] * y.wpc;
                     const uint32_t w[4] = {r[u].x, r[u].y, r[u].z, r[u].w};
 #pragma unroll
                     for (int e = 0; e < 8; e++) {
@@ -372,36 +376,41 @@ __global__ __launch_bounds__(NT) void traverse_block_kernel(QueryArgs a, BlockLa
                         atomicSub(&mcnt[local >> kFshift], 1u << ((local & (kFpw - 1u)) * CBITS));
                     }
                 }
-            } else {
-                // all atomics of the batch first, then the (rare) promotions: a compare
-                // right behind each returning atomic would serialise on LDS latency
-                uint32_t old[kUnroll][8];
+                return;
+            }
+            // all atomics of the batch first, then the (rare) promotions: a compare right
+            // behind each returning atomic would serialise on LDS latency
+            uint32_t old[kUnroll][8];
 #pragma unroll
-                for (int u = 0; u < kUnroll; u++) {
-                    if (sreg[u] < 0) continue;
-                    uint32_t* mcnt = cnt + (size_t)((sreg[u] >> 1) / a.L) * y.wpc;
-                    const uint32_t w[4] = {r[u].x, r[u].y, r[u].z, r[u].w};
+            for (int u = 0; u < kUnroll; u++) {
+                if (mr[u] < 0) continue;
+                uint32_t* mcnt = cnt + (size_t)mr[u] * y.wpc;
+                const uint32_t w[4] = {r[u].x, r[u].y, r[u].z, r[u].w};
 #pragma unroll
-                    for (int e = 0; e < 8; e++) {
-                        const uint32_t local = (w[e >> 1] >> ((e & 1) * 16)) & 0xffffu;
-                        old[u][e] = atomicAdd(&mcnt[local >> kFshift], 1u << ((local & (kFpw - 1u)) * CBITS));
-                    }
+                for (int e = 0; e < 8; e++) {
+                    const uint32_t local = (w[e >> 1] >> ((e & 1) * 16)) & 0xffffu;
+                    old[u][e] = atomicAdd(&mcnt[local >> kFshift], 1u << ((local & (kFpw - 1u)) * CBITS));
                 }
+            }
 #pragma unroll
-                for (int u = 0; u < kUnroll; u++) {
-                    if (sreg[u] < 0) continue;
-                    const uint32_t w[4] = {r[u].x, r[u].y, r[u].z, r[u].w};
+            for (int u = 0; u < kUnroll; u++) {
+                if (mr[u] < 0) continue;
+                const uint32_t w[4] = {r[u].x, r[u].y, r[u].z, r[u].w};
 #pragma unroll
-                    for (int e = 0; e < 8; e++) {
-                        const uint32_t local = (w[e >> 1] >> ((e & 1) * 16)) & 0xffffu;
-                        if (((old[u][e] >> ((local & (kFpw - 1u)) * CBITS)) & kCmask) == Lm1) {
-                            const uint32_t slot = atomicAdd(&misc[kPromoCount], 1u);
-                            if (slot < (uint32_t)kPromoCap)
-                                promo[slot] = local | ((uint32_t)((sreg[u] >> 1) / a.L) << 26);
-                        }
+                for (int e = 0; e < 8; e++) {
+                    const uint32_t local = (w[e >> 1] >> ((e & 1) * 16)) & 0xffffu;
+                    if (((old[u][e] >> ((local & (kFpw - 1u)) * CBITS)) & kCmask) == Lm1) {
+                        const uint32_t slot = atomicAdd(&misc[kPromoCount], 1u);
+                        if (slot < (uint32_t)kPromoCap) promo[slot] = local | ((uint32_t)mr[u] << 26);
                     }
                 }
             }
+        };
+        for (int g0 = 0; g0 < total; g0 += NT * kUnroll) {
+            uint4 r4[kUnroll];
+            int mr[kUnroll];
+            fetch(g0, r4, mr);
+            process(r4, mr);
         }
         unsigned long long streamed = 0;
         for (int s = 0; s < S; s++) streamed += (unsigned long long)max(0, s_rb[s] - s_ra[s]);
@@ -501,7 +510,10 @@ __global__ __launch_bounds__(NT) void traverse_block_kernel(QueryArgs a, BlockLa
             __syncthreads();
         }
         {
-            constexpr int kGroup = 32;
+            // Eight lanes rank one promotion, so 32 promotions are in flight per
+            // workgroup; each lane runs the binary searches of up to four streams in
+            // lockstep so that their key reads overlap.
+            constexpr int kGroup = 8, kPerLane = 4;
             const int gl = tid & (kGroup - 1);
             const int group = tid / kGroup;
             for (uint32_t pi = group; pi < np; pi += NT / kGroup) {
@@ -541,19 +553,59 @@ __global__ __launch_bounds__(NT) void traverse_block_kernel(QueryArgs a, BlockLa
                 }
                 // rank of that window = windows of the composite ordered before it
                 uint32_t rank = 0;
-                for (int s2 = gl; s2 < 2 * a.L; s2 += kGroup) {
-                    const int h2 = s2 >> 1, side2 = s2 & 1;
-                    const int sidx = 2 * (m * a.L + h2) + side2;
-                    int c;
-                    if (h2 == w_h) {
-                        const bool corner = s_p[m * a.L + h2] == n - 1 && T >= 2;  // ghost window first
-                        if (side2 == w_side) c = w_j;
-                        else if (corner) c = w_side ? 0 : s_ns[sidx];
-                        else c = count_in_epoch(sidx, w_bits, w_side == 0);
-                    } else {
-                        c = count_in_epoch(sidx, w_bits, h2 > w_h);
+                for (int s0 = gl; s0 < 2 * a.L; s0 += kGroup * kPerLane) {
+                    Stream st[kPerLane];
+                    int lo[kPerLane], hi[kPerLane];
+                    bool strict[kPerLane];
+#pragma unroll
+                    for (int u = 0; u < kPerLane; u++) {
+                        const int s2 = s0 + u * kGroup;
+                        lo[u] = hi[u] = 0;
+                        strict[u] = false;
+                        if (s2 >= 2 * a.L) continue;
+                        const int h2 = s2 >> 1, side2 = s2 & 1;
+                        const int sidx = 2 * (m * a.L + h2) + side2;
+                        st[u] = load_stream(sidx);
+                        if (h2 == w_h) {
+                            const bool corner = st[u].p == n - 1 && T >= 2;   // ghost window first
+                            if (side2 == w_side) { lo[u] = hi[u] = w_j; continue; }
+                            if (corner) { lo[u] = hi[u] = w_side ? 0 : s_ns[sidx]; continue; }
+                            strict[u] = w_side == 0;
+                        } else {
+                            strict[u] = h2 > w_h;
+                        }
+                        // the epoch's range, narrowed by the sampled priorities
+                        lo[u] = s_cprev[sidx]; hi[u] = s_c[sidx];
+                        const int len = hi[u] - lo[u];
+                        if (len >= 32) {
+                            const uint32_t* tab = s_samp + sidx * 16;
+                            int tl = 0, th = 15;
+                            while (tl < th) {
+                                const int mid = (tl + th + 1) >> 1;
+                                const uint32_t v = tab[mid];
+                                if (strict[u] ? v < w_bits : v <= w_bits) tl = mid; else th = mid - 1;
+                            }
+                            const int base0 = lo[u];
+                            if (tl > 0) lo[u] = base0 + (int)(((int64_t)len * tl) >> 4) + 1;
+                            if (tl < 15) hi[u] = base0 + (int)(((int64_t)len * (tl + 1)) >> 4);
+                        }
                     }
-                    rank += (uint32_t)c;
+                    for (;;) {
+                        bool any = false;
+#pragma unroll
+                        for (int u = 0; u < kPerLane; u++) {
+                            if (lo[u] < hi[u]) {
+                                any = true;
+                                const int mid = (lo[u] + hi[u]) >> 1;
+                                const uint32_t v = stream_prio_bits(st[u], mid);
+                                probes++;
+                                if (strict[u] ? v < w_bits : v <= w_bits) lo[u] = mid + 1; else hi[u] = mid;
+                            }
+                        }
+                        if (!any) break;
+                    }
+#pragma unroll
+                    for (int u = 0; u < kPerLane; u++) rank += (uint32_t)lo[u];
                 }
                 for (int o = kGroup / 2; o > 0; o >>= 1) rank += (uint32_t)__shfl_xor((int)rank, o, kGroup);
                 if (gl == 0) {
@@ -781,21 +833,22 @@ bool block_traversal_supported(const QueryArgs& a, size_t* lds_bytes) {
 
 int query_block(const QueryArgs& a, hipStream_t s) {
     const BlockLayout y = make_block_layout(a);
-    static bool attr_done = false;
-    if (!attr_done) {
-        DCIH_HIP(hipFuncSetAttribute((const void*)traverse_block_kernel<kBlockThreads, 4>,
-                                     hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024));
-        DCIH_HIP(hipFuncSetAttribute((const void*)traverse_block_kernel<kBlockThreads, 8>,
-                                     hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024));
-        attr_done = true;
-    }
     const int64_t items = (int64_t)a.nq * a.B;
-    if (y.cbits == 4)
-        hipLaunchKernelGGL((traverse_block_kernel<kBlockThreads, 4>), dim3((unsigned)items),
-                           dim3(kBlockThreads), y.lds_bytes, s, a, y);
-    else
-        hipLaunchKernelGGL((traverse_block_kernel<kBlockThreads, 8>), dim3((unsigned)items),
-                           dim3(kBlockThreads), y.lds_bytes, s, a, y);
+    const bool many = 160 * 1024 / y.lds_bytes >= 4;     // four or more workgroups per CU by LDS
+#define DCIH_LAUNCH(CB, MW)                                                                        \
+    do {                                                                                           \
+        static bool attr_done = false;                                                             \
+        if (!attr_done) {                                                                          \
+            DCIH_HIP(hipFuncSetAttribute((const void*)traverse_block_kernel<kBlockThreads, CB, MW>, \
+                                         hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024)); \
+            attr_done = true;                                                                      \
+        }                                                                                          \
+        hipLaunchKernelGGL((traverse_block_kernel<kBlockThreads, CB, MW>), dim3((unsigned)items),  \
+                           dim3(kBlockThreads), y.lds_bytes, s, a, y);                             \
+    } while (0)
+    if (y.cbits == 4) { if (many) DCIH_LAUNCH(4, 4); else DCIH_LAUNCH(4, 3); }
+    else              { if (many) DCIH_LAUNCH(8, 4); else DCIH_LAUNCH(8, 3); }
+#undef DCIH_LAUNCH
     DCIH_HIP(hipGetLastError());
     return 0;
 }
