@@ -5,7 +5,7 @@
 // result [num_indices][num_points]) and for the queries (:802-803).
 //
 // The contraction is thin (a few tens of directions), so every row is read
-// from HBM exactly once, staged through LDS in 32-column chunks with coalesced
+// from HBM exactly once, staged through LDS in 16-column chunks with coalesced
 // 16-byte loads, and each thread keeps one row's dot products with up to 32
 // directions in registers.  Direction values are wave-uniform and are fetched
 // through the scalar cache.  Output stores are coalesced along the row index.
@@ -17,8 +17,10 @@
 namespace dcih {
 
 constexpr int kProjRows = 256;    // rows per workgroup = threads per workgroup
-constexpr int kProjChunk = 32;    // columns staged per LDS tile
-constexpr int kProjStride = 36;   // LDS row pitch in floats (16 B aligned, conflict-free b128 reads)
+constexpr int kProjChunk = 16;    // columns staged per LDS tile
+constexpr int kProjStride = 20;   // LDS row pitch in floats (16 B aligned, conflict-free b128 reads)
+constexpr int kProjTpr = kProjChunk / 4;          // threads that cover one row's chunk with float4 loads
+constexpr int kProjRpp = kProjRows / kProjTpr;    // rows covered per pass of the workgroup
 
 template <int RT>
 __global__ __launch_bounds__(kProjRows) void project_kernel(
@@ -34,23 +36,33 @@ __global__ __launch_bounds__(kProjRows) void project_kernel(
 #pragma unroll
     for (int r = 0; r < RT; r++) acc[r] = 0.0f;
 
+    // The next chunk's global reads are issued into registers before the current
+    // chunk is consumed, so their latency hides behind the FMAs of this workgroup
+    // instead of leaving its waves parked at the barrier.
+    const int kq = (tid % kProjTpr) * 4;      // float4 path: kProjTpr threads cover one row's chunk
+    float4 pre[kProjRows / kProjRpp];
+    auto prefetch = [&](int k0) {
+        const int kc = min(kProjChunk, dim - k0);
+#pragma unroll
+        for (int j = 0; j < kProjRows / kProjRpp; j++) {
+            const int row = tid / kProjTpr + kProjRpp * j;
+            pre[j] = make_float4(0.f, 0.f, 0.f, 0.f);
+            if (row < rows_here && kq < kc)
+                pre[j] = *reinterpret_cast<const float4*>(rows + (row0 + row) * dim + k0 + kq);
+        }
+    };
+    if (vec4) prefetch(0);
     for (int k0 = 0; k0 < dim; k0 += kProjChunk) {
         const int kc = min(kProjChunk, dim - k0);
         __syncthreads();
         if (vec4) {
-            // 8 threads cover one row's 32 columns with float4 loads.
-            const int kq = (tid & 7) * 4;
 #pragma unroll
-            for (int j = 0; j < kProjRows / 32; j++) {
-                const int row = (tid >> 3) + 32 * j;
-                float4 v = make_float4(0.f, 0.f, 0.f, 0.f);
-                if (row < rows_here && kq < kc)
-                    v = *reinterpret_cast<const float4*>(rows + (row0 + row) * dim + k0 + kq);
-                *reinterpret_cast<float4*>(&tile[row * kProjStride + kq]) = v;
-            }
+            for (int j = 0; j < kProjRows / kProjRpp; j++)
+                *reinterpret_cast<float4*>(&tile[(tid / kProjTpr + kProjRpp * j) * kProjStride + kq]) = pre[j];
+            if (k0 + kProjChunk < dim) prefetch(k0 + kProjChunk);
         } else {
             for (int e = tid; e < kProjRows * kProjChunk; e += kProjRows) {
-                const int row = e >> 5, kk = e & 31;
+                const int row = e / kProjChunk, kk = e % kProjChunk;
                 float v = 0.f;
                 if (row < rows_here && kk < kc) v = rows[(row0 + row) * dim + k0 + kk];
                 tile[row * kProjStride + kk] = v;
