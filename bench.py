@@ -28,6 +28,7 @@ TUNED = {
     "c2": dict(bs=32, ts=4, outer=500),
     "c3": dict(bs=1000, ts=16, outer=500),
     "c4": dict(bs=100, ts=10, outer=500),
+    "c5": dict(bs=640, ts=2, outer=500),
 }
 
 
@@ -49,6 +50,7 @@ def parse():
     p.add_argument("--counter-queries", type=int, default=512,
                    help="queries whose exact traversal counters are taken (step-by-step kernel)")
     p.add_argument("--traversal", default="auto", choices=["auto", "step", "batch"])
+    p.add_argument("--c5-batches", type=int, default=20, help="batches of the incremental workload")
     p.add_argument("--copy-calibration", action="store_true",
                    help="also run a plain 1 GiB device copy (known HBM traffic) so that "
                         "rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE readings can be scaled")
@@ -72,6 +74,59 @@ def recall_at_k(ids, gt):
     return hit / gt.numel()
 
 
+def run_c5(a):
+    """Incremental workload: batches of 1M x 64 N(0,1) rows appended one after the
+    other, the fixed query batch run after each; one JSON line with per-size figures."""
+    import numpy as np
+    import torch
+    import dciknn_cuda_amd as D
+    from dciknn_cuda_amd import workloads
+    cfg = dict(TUNED["c5"])
+    for key in ("bs", "ts", "outer"):
+        if getattr(a, key) is not None:
+            cfg[key] = getattr(a, key)
+    shape = workloads.SHAPES[5]
+    n_batch = a.n or shape["n"]
+    nq = a.nq or shape["nq"]
+    M, L, k, dim = shape["m"], shape["l"], shape["k"], 64
+    Qd = workloads.c5_queries(nq).cuda()
+    dci = D.DCI(dim, M, L, cfg["bs"], cfg["ts"], seed=4)
+    rows = []
+    all_x = []
+    for b in range(a.c5_batches):
+        xb = workloads.c5_batch(b, n=n_batch).cuda()
+        all_x.append(xb)
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        dci.append(xb)
+        torch.cuda.synchronize()
+        t_add = time.perf_counter() - t0
+        dci.query(Qd, k, cfg["outer"], return_int=True)          # warm-up (hints, workspace)
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        ids, dists = dci.query(Qd, k, cfg["outer"], return_int=True)
+        torch.cuda.synchronize()
+        t_q = time.perf_counter() - t0
+        X = torch.cat(all_x)
+        gt = exact_knn_gpu(X, Qd[:256], k)
+        rec = recall_at_k(ids[:256].long(), gt)
+        del X
+        rows.append(dict(points=dci.num_points, append_ms=t_add * 1e3,
+                         new_points_per_s=n_batch / t_add, total_points_per_s=dci.num_points / t_add,
+                         queries_per_s=nq / t_q, recall_at_k=rec))
+    out = {"metric": "queries/sec; index build points/sec (incremental)", "value": rows[-1]["queries_per_s"],
+           "unit": "queries/s", "n_gpus": 1, "steps": 1, "warmup": 1,
+           "ms_per_step": nq / rows[-1]["queries_per_s"] * 1e3, "higher_is_better": True,
+           "scaling": "weak", "vs_baseline": None, "dtype": "f32", "data": "synthetic",
+           "config": {"workload": "C5: %d appends of %d x 64 fp32 N(0,1), %d queries, m=%d L=%d k=%d"
+                                  % (a.c5_batches, n_batch, nq, M, L, k),
+                      "block_size": cfg["bs"], "thread_size": cfg["ts"],
+                      "num_outer_iterations": cfg["outer"]},
+           "build_points_per_s": rows[-1]["total_points_per_s"], "per_size": rows,
+           "roofline": None, "cpu_baseline": None}
+    print(json.dumps(out))
+
+
 def main():
     a = parse()
     if a.gpus != 1:
@@ -86,6 +141,8 @@ def main():
     import dciknn_cuda_amd as D
     from dciknn_cuda_amd import _capi, workloads
 
+    if a.config == "c5":
+        return run_c5(a)
     cfg = dict(TUNED[a.config])
     for key in ("bs", "ts", "outer"):
         if getattr(a, key) is not None:

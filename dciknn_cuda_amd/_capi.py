@@ -27,6 +27,8 @@ SIGNATURES = {
     "dcih_set_directions": (_c.c_int, [_c.c_void_p, _c.c_void_p]),
     "dcih_add": (_c.c_int, [_c.c_void_p, _c.c_int, _c.c_int64, _c.c_void_p, _c.c_int,
                             _c.c_int, _c.c_void_p]),
+    "dcih_append": (_c.c_int, [_c.c_void_p, _c.c_int, _c.c_int64, _c.c_void_p, _c.c_int,
+                               _c.c_int, _c.c_void_p]),
     "dcih_query": (_c.c_int, [_c.c_void_p, _c.c_int, _c.c_int, _c.c_void_p, _c.c_int,
                               _c.c_int, _c.c_int, _c.c_int, _c.c_int, _c.c_int,
                               _c.c_void_p, _c.c_void_p, _c.c_void_p, _c.c_void_p]),

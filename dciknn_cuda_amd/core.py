@@ -123,6 +123,20 @@ class DCI(object):
         self.num_points = data.shape[0]
         self._array = data   # the index borrows this memory
 
+    def append(self, data):
+        """Insert more rows (not in the reference, whose `add` works once): the
+        index becomes what `add` would build over all rows given so far; ids
+        continue after the existing ones.  The rows are copied."""
+        self._require_handle()
+        self._check_data(data)
+        if data.device != self._device:
+            raise ValueError("tensor is on %s but this DCI instance lives on %s" % (data.device, self._device))
+        _capi.check(self._lib.dcih_append(self._dci_inst, self._dim, data.shape[0], data.data_ptr(),
+                                          self._block_size, self._thread_size,
+                                          _stream_ptr(self._device)))
+        self.num_points += data.shape[0]
+        self._array = None    # the index owns its rows now
+
     # query is num_queries x dim, returns num_queries x num_neighbours
     def query(self, query, num_neighbours=-1, num_outer_iterations=5000, blind=False,
               *, return_int=False, return_counters=False):

@@ -89,6 +89,8 @@ struct dcih_index {
     int32_t* d_sids = nullptr;          // [I][n]
     uint32_t* d_inv = nullptr;          // [I][n] position of each point in its sorted slice
     uint16_t* d_lids = nullptr;         // [I][n] partition-relative ids (partitions <= 65536 points)
+    float* d_own = nullptr;             // rows copied in by dcih_append (the index owns these)
+    int64_t own_rows = 0;               // capacity of d_own in rows
     float* d_stop_hint = nullptr;       // [block_size] epoch-size hints learnt from earlier queries
     int hint_k = 0, hint_outer = 0, hint_T = 0, hint_maxc = 0;   // query shape the hints belong to
     int traversal = 0;                  // DCIH_OPT_TRAVERSAL value
@@ -127,16 +129,23 @@ int draw_directions(dcih_index* h) {
     return 0;
 }
 
-int release_index(dcih_index* h) {
+// Frees the sorted arrays but keeps the rows.
+int release_sorted(dcih_index* h) {
     if (h->d_skeys) { DCIH_HIP(hipFree(h->d_skeys)); h->d_skeys = nullptr; }
     if (h->d_sids) { DCIH_HIP(hipFree(h->d_sids)); h->d_sids = nullptr; }
     if (h->d_inv) { DCIH_HIP(hipFree(h->d_inv)); h->d_inv = nullptr; }
     if (h->d_lids) { DCIH_HIP(hipFree(h->d_lids)); h->d_lids = nullptr; }
     if (h->d_stop_hint) { DCIH_HIP(hipFree(h->d_stop_hint)); h->d_stop_hint = nullptr; }
+    return 0;
+}
+
+int release_index(dcih_index* h) {
+    const int rc = release_sorted(h);
+    if (h->d_own) { (void)hipFree(h->d_own); h->d_own = nullptr; h->own_rows = 0; }
     h->d_data = nullptr;
     h->n = 0;
     h->block_size = 0;
-    return 0;
+    return rc;
 }
 
 int ensure_ws(dcih_index* h, size_t bytes) {
@@ -207,18 +216,12 @@ int dcih_set_directions(dcih_index* h, const float* h_dirs) {
     return DCIH_OK;
 }
 
-int dcih_add(dcih_index* h, int dim, int64_t num_points, const float* d_data,
-             int block_size, int thread_size, void* stream) {
-    if (!h) return fail(DCIH_EINVAL, "dcih_add: null handle");
-    if (dim != h->dim) return fail(DCIH_EINVAL, "dcih_add: dim differs from the index's");
-    if (h->n > 0) return fail(DCIH_ESTATE, "dcih_add: index already holds points; clear it first");
-    if (num_points <= 0 || !d_data) return fail(DCIH_EINVAL, "dcih_add: no points given");
-    if (num_points > 0x7fffffffLL) return fail(DCIH_EINVAL, "dcih_add: more than 2^31-1 points");
-    if (block_size <= 0 || thread_size <= 0)
-        return fail(DCIH_EINVAL, "dcih_add: block_size and thread_size must be positive");
-    DeviceGuard guard(h->device);
-    hipStream_t s = (hipStream_t)stream;
+// Projects and sorts `num_points` rows at d_data into a fresh index (the handle holds
+// no sorted arrays when this is called).  Synchronises the stream before returning.
+static int build_index(dcih_index* h, int64_t num_points, const float* d_data, int block_size,
+                       hipStream_t s) {
     const int I = num_indices(h);
+    const int dim = h->dim;
     const size_t cells = (size_t)I * num_points;
     float* d_keys = nullptr;
     void* d_tmp = nullptr;
@@ -234,11 +237,11 @@ int dcih_add(dcih_index* h, int dim, int64_t num_points, const float* d_data,
             hipMalloc(&h->d_stop_hint, (size_t)block_size * sizeof(float)) != hipSuccess ||
             hipMalloc(&d_keys, cells * sizeof(float)) != hipSuccess ||
             (tmp_bytes && hipMalloc(&d_tmp, tmp_bytes) != hipSuccess)) {
-            rc = fail(DCIH_EHIP, "dcih_add: out of device memory");
+            rc = fail(DCIH_EHIP, "build: out of device memory");
             break;
         }
         if (hipMemsetAsync(h->d_stop_hint, 0, (size_t)block_size * sizeof(float), s) != hipSuccess) {
-            rc = fail(DCIH_EHIP, "dcih_add: clearing the hint table failed");
+            rc = fail(DCIH_EHIP, "build: clearing the hint table failed");
             break;
         }
         mark(h, DCIH_T_PROJECT, 0, s);
@@ -254,12 +257,67 @@ int dcih_add(dcih_index* h, int dim, int64_t num_points, const float* d_data,
     if (d_keys) (void)hipFree(d_keys);
     if (d_tmp) (void)hipFree(d_tmp);
     if (rc == DCIH_OK && se != hipSuccess)
-        rc = fail(DCIH_EHIP, std::string("dcih_add: ") + hipGetErrorString(se));
-    if (rc) { (void)release_index(h); return rc; }
+        rc = fail(DCIH_EHIP, std::string("build: ") + hipGetErrorString(se));
+    if (rc) return rc;
     h->d_data = d_data;
     h->n = num_points;
     h->block_size = block_size;
+    h->hint_k = h->hint_outer = h->hint_T = h->hint_maxc = 0;
     return DCIH_OK;
+}
+
+int dcih_add(dcih_index* h, int dim, int64_t num_points, const float* d_data,
+             int block_size, int thread_size, void* stream) {
+    if (!h) return fail(DCIH_EINVAL, "dcih_add: null handle");
+    if (dim != h->dim) return fail(DCIH_EINVAL, "dcih_add: dim differs from the index's");
+    if (h->n > 0) return fail(DCIH_ESTATE, "dcih_add: index already holds points; clear it first");
+    if (num_points <= 0 || !d_data) return fail(DCIH_EINVAL, "dcih_add: no points given");
+    if (num_points > 0x7fffffffLL) return fail(DCIH_EINVAL, "dcih_add: more than 2^31-1 points");
+    if (block_size <= 0 || thread_size <= 0)
+        return fail(DCIH_EINVAL, "dcih_add: block_size and thread_size must be positive");
+    DeviceGuard guard(h->device);
+    const int rc = build_index(h, num_points, d_data, block_size, (hipStream_t)stream);
+    if (rc) (void)release_index(h);
+    return rc;
+}
+
+int dcih_append(dcih_index* h, int dim, int64_t num_points, const float* d_data,
+                int block_size, int thread_size, void* stream) {
+    if (!h) return fail(DCIH_EINVAL, "dcih_append: null handle");
+    if (dim != h->dim) return fail(DCIH_EINVAL, "dcih_append: dim differs from the index's");
+    if (num_points <= 0 || !d_data) return fail(DCIH_EINVAL, "dcih_append: no points given");
+    if (block_size <= 0 || thread_size <= 0)
+        return fail(DCIH_EINVAL, "dcih_append: block_size and thread_size must be positive");
+    if (h->n > 0 && block_size != h->block_size)
+        return fail(DCIH_EINVAL, "dcih_append: block_size differs from the one the index was built with");
+    const int64_t total = h->n + num_points;
+    if (total > 0x7fffffffLL) return fail(DCIH_EINVAL, "dcih_append: more than 2^31-1 points");
+    DeviceGuard guard(h->device);
+    hipStream_t s = (hipStream_t)stream;
+    const size_t row_bytes = (size_t)dim * sizeof(float);
+    // all rows move into one buffer the index owns (capacity doubles, so copies amortise)
+    if (!h->d_own || h->own_rows < total) {
+        const int64_t cap = std::max<int64_t>(total, 2 * h->own_rows);
+        float* fresh = nullptr;
+        DCIH_HIP(hipMalloc(&fresh, (size_t)cap * row_bytes));
+        if (h->n > 0)
+            DCIH_HIP(hipMemcpyAsync(fresh, h->d_data, (size_t)h->n * row_bytes, hipMemcpyDeviceToDevice, s));
+        DCIH_HIP(hipStreamSynchronize(s));
+        if (h->d_own) (void)hipFree(h->d_own);
+        h->d_own = fresh;
+        h->own_rows = cap;
+    } else if (h->n > 0 && h->d_data != h->d_own) {
+        DCIH_HIP(hipMemcpyAsync(h->d_own, h->d_data, (size_t)h->n * row_bytes, hipMemcpyDeviceToDevice, s));
+    }
+    DCIH_HIP(hipMemcpyAsync(h->d_own + (size_t)h->n * dim, d_data, (size_t)num_points * row_bytes,
+                            hipMemcpyDeviceToDevice, s));
+    // the partition boundaries move with the total, so every slice is rebuilt
+    DCIH_HIP(hipStreamSynchronize(s));
+    int rc = release_sorted(h);
+    if (rc) return rc;
+    rc = build_index(h, total, h->d_own, block_size, s);
+    if (rc) (void)release_index(h);
+    return rc;
 }
 
 int dcih_query(dcih_index* h, int dim, int num_queries, const float* d_query,

@@ -102,6 +102,19 @@ int dcih_add(dcih_index* h, int dim, int64_t num_points, const float* d_data,
              int block_size, int thread_size, void* stream);
 
 /*
+ * Incremental insertion; no counterpart in the reference, which refuses a second
+ * add (dciknn_cuda/core.py:70-71, src/dci_cuda_kernel.cu:157).  The result is
+ * exactly the index dcih_add would build over all rows given so far, in the order
+ * given (ids continue where the previous call stopped).  Unlike dcih_add the rows
+ * are COPIED into a buffer the index owns, so d_data may be released after the
+ * call; rows of an earlier dcih_add are copied as well.  The partition boundaries
+ * depend on the total, so every slice is projected and sorted again.  Synchronises
+ * the stream.
+ */
+int dcih_append(dcih_index* h, int dim, int64_t num_points, const float* d_data,
+                int block_size, int thread_size, void* stream);
+
+/*
  * Replaces dci_query (include/dci.h:71, src/dci_cuda_kernel.cu:777-875) with
  * query_config.blind == false.  d_query is [num_queries][dim]; for each query
  * d_nn / d_dists [num_queries][num_neighbours] receive the ids and Euclidean

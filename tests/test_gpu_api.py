@@ -148,3 +148,46 @@ def test_non_default_stream(gpu, oracle):
     s.synchronize()
     i0, d0 = dci.query(Q, 5, 30)
     assert torch.equal(i0, i1) and torch.equal(d0, d1)
+
+
+def test_append_equals_one_add_of_the_concatenation(gpu, oracle):
+    """Incremental insertion is defined as 'as if built on all rows so far'."""
+    g = torch.Generator().manual_seed(3)
+    X = torch.randn(9000, 24, generator=g).cuda()
+    Q = torch.randn(40, 24, generator=g).cuda()
+    whole = gpu.DCI(24, 2, 4, 6, 5, seed=9)
+    whole.add(X)
+    want = whole.query(Q, 8, 40, return_int=True)
+    parts = gpu.DCI(24, 2, 4, 6, 5, seed=9)
+    parts.add(X[:2500].contiguous())                  # a borrowed first batch ...
+    with pytest.raises(RuntimeError):
+        parts.add(X[2500:5000].contiguous())          # ... `add` still works only once
+    cuts = [2500, 2501, 6000, 9000]
+    for lo, hi in zip(cuts[:-1], cuts[1:]):
+        chunk = X[lo:hi].clone()
+        parts.append(chunk)
+        del chunk                                     # appended rows are copied
+        assert parts.num_points == hi
+        torch.cuda.synchronize()
+        ref = gpu.DCI(24, 2, 4, 6, 5, seed=9)
+        ref.add(X[:hi].contiguous())
+        a = parts.query(Q, 8, 40, return_int=True)
+        b = ref.query(Q, 8, 40, return_int=True)
+        assert torch.equal(a[0], b[0]) and torch.equal(a[1], b[1])
+        ref.free()
+    got = parts.query(Q, 8, 40, return_int=True)
+    assert torch.equal(got[0], want[0]) and torch.equal(got[1], want[1])
+    # and the oracle on the concatenation agrees
+    r = oracle.knn(parts.directions.numpy(), X.cpu().numpy(), Q.cpu().numpy(), 2, 4, 6, 5, 8, 40)
+    assert np.array_equal(got[0].cpu().numpy(), r["ids"])
+    # append on an empty index, then clear
+    fresh = gpu.DCI(24, 2, 4, 6, 5, seed=9)
+    fresh.append(X[:100].contiguous())
+    fresh.append(X[100:9000].contiguous())
+    c = fresh.query(Q, 8, 40, return_int=True)
+    assert torch.equal(c[0], want[0]) and torch.equal(c[1], want[1])
+    fresh.clear()
+    assert fresh.num_points == 0
+    fresh.add(X)
+    d = fresh.query(Q, 8, 40, return_int=True)
+    assert torch.equal(d[0], want[0])
