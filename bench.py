@@ -21,6 +21,14 @@ sys.path.insert(0, ROOT)
 
 HBM_PEAK_GBS = 8000.0   # MI355X HBM3E
 
+# HBM bytes per launch of the batch traversal kernel on the default workload and
+# setting (C2 at TUNED["c2"], all 10000 queries), from rocprofv3 --pmc FETCH_SIZE and
+# WRITE_SIZE, each scaled by what the same counter reads for a 1 GiB device copy
+# (2.000 and 1.000); the counter runs are summarised in profiles/bench_c2_hbm_traffic.txt.
+# Counters cannot be read from inside this process, so the figure is a constant
+# tied to that exact configuration and omitted for any other.
+MEASURED_TRAFFIC_C2_DEFAULT = 373.8e9
+
 # (block_size, thread_size, num_outer_iterations) used when none are given:
 # the fastest setting found with recall@k >= 0.95 on that workload.
 TUNED = {
@@ -235,8 +243,11 @@ def main():
     trav_avg_ms = float(np.mean(trav_ms))
     achieved = bytes_per_query * nq / (trav_avg_ms * 1e-3) / 1e9
     kernel = "traverse_kernel" if a.traversal == "step" else "traverse_block_kernel"
+    default_run = (a.config == "c2" and cfg == TUNED["c2"] and a.traversal == "auto"
+                   and N == workloads.SHAPES[2]["n"] and nq == workloads.SHAPES[2]["nq"])
     roofline = dict(bound="hbm", kernel=kernel, achieved=achieved, peak=HBM_PEAK_GBS,
-                    unit="GB/s", frac=achieved / HBM_PEAK_GBS, traffic=None,
+                    unit="GB/s", frac=achieved / HBM_PEAK_GBS,
+                    traffic=MEASURED_TRAFFIC_C2_DEFAULT if default_run else None,
                     bytes_per_launch=bytes_per_query * nq, avg_launch_ms=trav_avg_ms,
                     own_layout_bytes_per_launch=bytes_own * nq,
                     own_layout_gbs=bytes_own * nq / (trav_avg_ms * 1e-3) / 1e9)
