@@ -95,9 +95,13 @@ struct dcih_index {
     int hint_k = 0, hint_outer = 0, hint_T = 0, hint_maxc = 0;   // query shape the hints belong to
     int traversal = 0;                  // DCIH_OPT_TRAVERSAL value
     unsigned long long* d_phase_ticks = nullptr;   // optional profile of the batch kernel
-    // grow-only query workspace
+    // grow-only workspace: query scratch, and the unsorted keys during a build
     void* ws = nullptr;
     size_t ws_bytes = 0;
+    // grow-only arena the sorted arrays and the hint table are carved from; kept
+    // across dcih_clear so that a rebuild allocates nothing
+    void* arena = nullptr;
+    size_t arena_bytes = 0;
     // optional per-kernel timing: ev[2*t], ev[2*t+1] bracket timer t
     bool profiling = false;
     hipEvent_t ev[2 * DCIH_NUM_TIMERS] = {};
@@ -129,13 +133,19 @@ int draw_directions(dcih_index* h) {
     return 0;
 }
 
-// Frees the sorted arrays but keeps the rows.
+// Drops the sorted arrays (their arena stays allocated for the next build) but keeps the rows.
 int release_sorted(dcih_index* h) {
-    if (h->d_skeys) { DCIH_HIP(hipFree(h->d_skeys)); h->d_skeys = nullptr; }
-    if (h->d_sids) { DCIH_HIP(hipFree(h->d_sids)); h->d_sids = nullptr; }
-    if (h->d_inv) { DCIH_HIP(hipFree(h->d_inv)); h->d_inv = nullptr; }
-    if (h->d_lids) { DCIH_HIP(hipFree(h->d_lids)); h->d_lids = nullptr; }
-    if (h->d_stop_hint) { DCIH_HIP(hipFree(h->d_stop_hint)); h->d_stop_hint = nullptr; }
+    h->d_skeys = nullptr;
+    h->d_sids = nullptr;
+    h->d_inv = nullptr;
+    h->d_lids = nullptr;
+    h->d_stop_hint = nullptr;
+    return 0;
+}
+
+int release_arena(dcih_index* h) {
+    (void)release_sorted(h);
+    if (h->arena) { DCIH_HIP(hipFree(h->arena)); h->arena = nullptr; h->arena_bytes = 0; }
     return 0;
 }
 
@@ -157,6 +167,14 @@ int ensure_ws(dcih_index* h, size_t bytes) {
 }
 
 size_t align_up(size_t v) { return (v + 255) & ~(size_t)255; }
+
+int ensure_arena(dcih_index* h, size_t bytes) {
+    if (bytes <= h->arena_bytes) return 0;
+    if (h->arena) { DCIH_HIP(hipFree(h->arena)); h->arena = nullptr; h->arena_bytes = 0; }
+    DCIH_HIP(hipMalloc(&h->arena, bytes));
+    h->arena_bytes = bytes;
+    return 0;
+}
 
 // Records the start (which = 0) or end (1) event of timer t when profiling.
 void mark(dcih_index* h, int t, int which, hipStream_t s) {
@@ -223,23 +241,28 @@ static int build_index(dcih_index* h, int64_t num_points, const float* d_data, i
     const int I = num_indices(h);
     const int dim = h->dim;
     const size_t cells = (size_t)I * num_points;
-    float* d_keys = nullptr;
-    void* d_tmp = nullptr;
     const size_t tmp_bytes = segsort_tmp_bytes(I, num_points, block_size);
     const bool small_parts = (num_points + block_size - 1) / block_size <= 65536;
-    int rc = DCIH_OK;
+    // one arena for what the index keeps, the workspace for what only the build needs:
+    // a rebuild of the same size allocates and frees nothing
+    const size_t b_keys = align_up(cells * sizeof(float));
+    const size_t b_ids = align_up(cells * sizeof(int32_t));
+    // +16: the traversal reads whole aligned 16-byte chunks, also at the very end
+    const size_t b_lids = small_parts ? align_up((cells + 16) * sizeof(uint16_t)) : 0;
+    const size_t b_hint = align_up((size_t)block_size * sizeof(float));
+    int rc = ensure_arena(h, 3 * b_keys + b_lids + b_hint);
+    if (rc) return rc;
+    rc = ensure_ws(h, b_keys + align_up(tmp_bytes));
+    if (rc) return rc;
+    char* base = (char*)h->arena;
+    h->d_skeys = (float*)base;
+    h->d_sids = (int32_t*)(base + b_keys);
+    h->d_inv = (uint32_t*)(base + b_keys + b_ids);
+    h->d_lids = small_parts ? (uint16_t*)(base + 3 * b_keys) : nullptr;
+    h->d_stop_hint = (float*)(base + 3 * b_keys + b_lids);
+    float* d_keys = (float*)h->ws;
+    void* d_tmp = tmp_bytes ? (void*)((char*)h->ws + b_keys) : nullptr;
     do {
-        if (hipMalloc(&h->d_skeys, cells * sizeof(float)) != hipSuccess ||
-            hipMalloc(&h->d_sids, cells * sizeof(int32_t)) != hipSuccess ||
-            hipMalloc(&h->d_inv, cells * sizeof(uint32_t)) != hipSuccess ||
-            // +16: the traversal reads whole aligned 16-byte chunks, also at the very end
-            (small_parts && hipMalloc(&h->d_lids, (cells + 16) * sizeof(uint16_t)) != hipSuccess) ||
-            hipMalloc(&h->d_stop_hint, (size_t)block_size * sizeof(float)) != hipSuccess ||
-            hipMalloc(&d_keys, cells * sizeof(float)) != hipSuccess ||
-            (tmp_bytes && hipMalloc(&d_tmp, tmp_bytes) != hipSuccess)) {
-            rc = fail(DCIH_EHIP, "build: out of device memory");
-            break;
-        }
         if (hipMemsetAsync(h->d_stop_hint, 0, (size_t)block_size * sizeof(float), s) != hipSuccess) {
             rc = fail(DCIH_EHIP, "build: clearing the hint table failed");
             break;
@@ -252,10 +275,8 @@ static int build_index(dcih_index* h, int64_t num_points, const float* d_data, i
         rc = segsort(d_keys, I, num_points, block_size, h->d_skeys, h->d_sids, h->d_inv, h->d_lids, d_tmp, s);
         mark(h, DCIH_T_SEGSORT, 1, s);
     } while (0);
-    // the scratch buffers are in use until the stream drains
+    // like the reference's dci_add, the call returns when the index is complete
     const hipError_t se = hipStreamSynchronize(s);
-    if (d_keys) (void)hipFree(d_keys);
-    if (d_tmp) (void)hipFree(d_tmp);
     if (rc == DCIH_OK && se != hipSuccess)
         rc = fail(DCIH_EHIP, std::string("build: ") + hipGetErrorString(se));
     if (rc) return rc;
@@ -464,6 +485,7 @@ int dcih_free(dcih_index* h) {
     DeviceGuard guard(h->device);
     (void)hipDeviceSynchronize();
     (void)release_index(h);
+    (void)release_arena(h);
     if (h->ws) (void)hipFree(h->ws);
     if (h->d_dirs) (void)hipFree(h->d_dirs);
     for (auto& e : h->ev) if (e) (void)hipEventDestroy(e);

@@ -162,7 +162,12 @@ int dcih_phase_profile(dcih_index* h, uint64_t* d_ticks);
 /* Number of points currently indexed (0 when empty). */
 int64_t dcih_num_points(const dcih_index* h);
 
-/* Replaces dci_clear (include/dci.h:77, src/dci_cuda_kernel.cu:878-885). */
+/*
+ * Replaces dci_clear (include/dci.h:77, src/dci_cuda_kernel.cu:878-885).  The
+ * index becomes empty; the device memory its arrays occupied stays with the
+ * handle, so that the next dcih_add allocates nothing, and is returned by
+ * dcih_free.
+ */
 int dcih_clear(dcih_index* h);
 
 /*
