@@ -242,13 +242,17 @@ __global__ __launch_bounds__(NT, MINW) void traverse_block_kernel(QueryArgs a, B
     // count: a composite left behind would keep the promotions of the others
     // waiting.  The total doubles from epoch to epoch until one has to be undone.
     // hint = running average of the step at which earlier queries stopped in this
-    // partition; it only steers epoch sizes (first jump to 3/4 of it, then +12 %
-    // per epoch), never results.
+    // partition; it only steers epoch sizes, never results.  The first jump goes
+    // 20 % past it: stop steps of one partition scatter little, so most items then
+    // finish in one or two epochs, and an epoch's fixed cost (bound search, ranking
+    // and replay round trips) outweighs the entries streamed past the stop step.
+    // Much further and the surplus promotions overflow the tables and force undos.
+    constexpr float kHintFirst = 1.2f, kHintGrow = 1.06f;
     const float hint = a.stop_hint ? a.stop_hint[b] : 0.0f;
     {
         int first = 4;
         for (int s = 0; s < S; s++) first = max(first, s_ns[s] / 128);
-        if (hint > 0.0f) first = max(first, (int)(0.75f * hint / (float)(2 * a.L)));
+        if (hint > 0.0f) first = max(first, (int)(kHintFirst * hint / (float)(2 * a.L)));
         if (tid < S) s_stride[tid] = first;
         if (tid < a.M) s_Kprev[tid] = 0;
     }
@@ -738,7 +742,7 @@ __global__ __launch_bounds__(NT, MINW) void traverse_block_kernel(QueryArgs a, B
                 const float t_armed = (float)(((unsigned long long)misc[kArmedHi] << 32) | misc[kArmedLo]);
                 k_target = fmaxf(t_armed + 1.0f, need) + (float)S;
             } else if (hint > 0.0f) {
-                k_target = (float)kmax < 0.7f * hint ? 0.75f * hint : 1.12f * (float)kmax + (float)S;
+                k_target = (float)kmax < 0.9f * kHintFirst * hint ? kHintFirst * hint : kHintGrow * (float)kmax + (float)S;
             }
             k_target = fminf(k_target, 2.0f * (float)kmax + 16.0f * (float)S);
             if (shrunk) k_target = fminf(k_target, (float)kmax + (float)dk_lead);
