@@ -33,7 +33,7 @@ MEASURED_TRAFFIC_C2_DEFAULT = 373.8e9
 # the fastest setting found with recall@k >= 0.95 on that workload.
 TUNED = {
     "c1": dict(bs=100, ts=10, outer=5000),
-    "c2": dict(bs=44, ts=3, outer=500),
+    "c2": dict(bs=56, ts=2, outer=500),
     "c3": dict(bs=1000, ts=16, outer=500),
     "c4": dict(bs=100, ts=10, outer=500),
     "c5": dict(bs=640, ts=2, outer=500),

@@ -39,7 +39,7 @@ namespace dcih {
 namespace {
 
 constexpr int kPromoCap = 256;      // promotions one epoch may produce
-constexpr int kPromoMax = 96;       // above this an epoch is undone and halved
+constexpr int kPromoMax = 160;       // above this an epoch is undone and halved
 constexpr int kMaxEpochs = 100000;
 constexpr uint32_t kInfBits = 0x7f800000u;
 
@@ -53,7 +53,7 @@ struct BlockLayout {
     int off_idx;      // per simple index: p, qp            (2 * I words)
     int off_stream;   // per stream: consumed, previous, total, range lo/hi, chunks, pos0, prefix (10 * 2I + 1 words, incl. stride and composite number)
     int off_chunk0;   // per stream: global index of its first 16-byte chunk (2I 64-bit words)
-    int off_comp;     // per composite: rho bits, K, active, previous K (4 * M words)
+    int off_comp;     // per composite: rho bits, K, active, previous K, sum of inverse priorities (5 * M words)
     int off_q;        // query row
     int off_samp;     // per stream: 16 sampled window priorities of the current epoch's range
     int off_promo, off_events, off_acc, off_sort, off_cnt;
@@ -63,7 +63,8 @@ struct BlockLayout {
 };
 
 __host__ __device__ inline int counter_bits_of(int L) {
-    return L <= 15 ? 4 : (L <= 255 ? 8 : (L <= 65535 ? 16 : 32));
+    // the all-ones value of a field marks a point already promoted, so L stays below it
+    return L <= 14 ? 4 : (L <= 254 ? 8 : (L <= 65534 ? 16 : 32));
 }
 
 BlockLayout make_block_layout(const QueryArgs& a) {
@@ -79,7 +80,7 @@ BlockLayout make_block_layout(const QueryArgs& a) {
     y.off_stream = o;   o += (10 * 2 * I + 2) * 4;
     o = (o + 7) & ~7;
     y.off_chunk0 = o;   o += 2 * I * 8;
-    y.off_comp = o;     o += 4 * a.M * 4;
+    y.off_comp = o;     o += 5 * a.M * 4;
     y.off_q = o;        o += ((a.dim + 3) & ~3) * 4;
     // small tables keep more workgroups resident per CU; an item that overflows them
     // is redone by the step-by-step kernel
@@ -174,6 +175,7 @@ __global__ __launch_bounds__(NT, MINW) void traverse_block_kernel(QueryArgs a, B
     uint32_t* s_K = s_rho + a.M;
     uint32_t* s_active = s_K + a.M;
     uint32_t* s_Kprev = s_active + a.M;
+    float* s_hsum = reinterpret_cast<float*>(s_Kprev + a.M);
     float* s_q = reinterpret_cast<float*>(smem + y.off_q);
     uint32_t* s_samp = reinterpret_cast<uint32_t*>(smem + y.off_samp);
     uint32_t* promo = reinterpret_cast<uint32_t*>(smem + y.off_promo);
@@ -242,12 +244,18 @@ __global__ __launch_bounds__(NT, MINW) void traverse_block_kernel(QueryArgs a, B
     // count: a composite left behind would keep the promotions of the others
     // waiting.  The total doubles from epoch to epoch until one has to be undone.
     // hint = running average of the step at which earlier queries stopped in this
-    // partition; it only steers epoch sizes, never results.  The first jump goes
-    // 20 % past it: stop steps of one partition scatter little, so most items then
-    // finish in one or two epochs, and an epoch's fixed cost (bound search, ranking
-    // and replay round trips) outweighs the entries streamed past the stop step.
-    // Much further and the surplus promotions overflow the tables and force undos.
-    constexpr float kHintFirst = 1.2f, kHintGrow = 1.06f;
+    // partition; it only steers epoch sizes, never results.  The first jump aims
+    // 5 % past it.  The number of points whose counters are complete grows like a
+    // high power (L) of the steps taken, so stop steps of one partition scatter
+    // little and most items finish in one or two epochs, while a jump 20 % too far
+    // already brings several times the promotions needed and overflows the tables.
+    // Where the stop needs more promotions than one epoch may produce (about
+    // k * T, against kPromoMax), the jump is shortened by the same power law so
+    // that an epoch yields about 0.6 * kPromoMax of them.
+    constexpr float kHintGrow = 1.06f, kPromoAim = 0.6f * (float)kPromoMax;
+    const float inv_L = 1.0f / (float)a.L;
+    const float kHintFirst =
+        fminf(1.05f, powf(kPromoAim / fmaxf(1.0f, (float)a.k * (float)T), inv_L));
     const float hint = a.stop_hint ? a.stop_hint[b] : 0.0f;
     {
         int first = 4;
@@ -287,24 +295,47 @@ __global__ __launch_bounds__(NT, MINW) void traverse_block_kernel(QueryArgs a, B
     };
 
     // Adds (or, for undo, removes) the visits of windows [cprev, c) of all streams.
-    // The loop is bound by vector-ALU issue (about 8 instructions and one LDS
-    // atomic per visit), so it reads partition-relative 16-bit ids, eight per
-    // aligned 16-byte chunk, and keeps per-visit work to shift / mask / atomic /
-    // compare with compile-time field widths.  The whole-chunk interior of every
-    // stream's range is laid end to end: consecutive threads read consecutive
-    // chunks whatever stream they belong to, several reads in flight each.  The
-    // one or two partial chunks at the ends of a range are handled separately
-    // with masks.  Returns the entries streamed (same value on every thread).
-    auto visit = [&](uint32_t* __restrict__ mcnt, uint32_t local, int m, bool undo) {
+    // The loop is bound by vector-ALU issue, so it reads partition-relative 16-bit
+    // ids, eight per aligned 16-byte chunk, and keeps per-visit work to shift /
+    // mask / one LDS atomic without return value, with compile-time field widths;
+    // which counters reached L is found afterwards by one scan of the counter
+    // words (collect_promotions).  The whole-chunk interior of every stream's
+    // range is laid end to end: consecutive threads read consecutive chunks
+    // whatever stream they belong to, the next batch of reads in flight while the
+    // current one is counted.  The one or two partial chunks at the ends of a
+    // range are handled separately with masks.  Returns the entries streamed (same
+    // value on every thread).
+    auto visit = [&](uint32_t* __restrict__ mcnt, uint32_t local, bool undo) {
         const uint32_t sh = (local & (kFpw - 1u)) * CBITS;
-        if (undo) {
-            atomicSub(&mcnt[local >> kFshift], 1u << sh);
-        } else {
-            const uint32_t old = atomicAdd(&mcnt[local >> kFshift], 1u << sh);
-            if (((old >> sh) & kCmask) == Lm1) {
-                const uint32_t slot = atomicAdd(&misc[kPromoCount], 1u);
-                if (slot < (uint32_t)kPromoCap) promo[slot] = local | ((uint32_t)m << 26);
+        if (undo) atomicSub(&mcnt[local >> kFshift], 1u << sh);
+        else atomicAdd(&mcnt[local >> kFshift], 1u << sh);
+    };
+    // Counters that stand at exactly L belong to points promoted in this epoch:
+    // a point is visited once per simple index, so its counter never passes L, and
+    // promotions of earlier epochs were moved to the all-ones value when their
+    // epoch was accepted (mark_promotions).
+    auto collect_promotions = [&]() {
+        constexpr uint32_t kRep = CBITS == 4 ? 0x11111111u : 0x01010101u;
+        const uint32_t want = (uint32_t)a.L * kRep;
+        const int words = a.M * y.wpc;
+        for (int w = tid; w < words; w += NT) {
+            const uint32_t x = cnt[w] ^ want;                       // zero field <=> counter == L
+            if (((x - kRep) & ~x & (kRep << (CBITS - 1))) == 0u) continue;   // no zero field
+            const int m = w / y.wpc;
+            const uint32_t first = (uint32_t)(w - m * y.wpc) << kFshift;
+#pragma unroll
+            for (uint32_t f = 0; f < kFpw; f++) {
+                if (((x >> (f * CBITS)) & kCmask) == 0u) {
+                    const uint32_t slot = atomicAdd(&misc[kPromoCount], 1u);
+                    if (slot < (uint32_t)kPromoCap) promo[slot] = (first + f) | ((uint32_t)m << 26);
+                }
             }
+        }
+    };
+    auto mark_promotions = [&](uint32_t np) {
+        for (uint32_t j = tid; j < np; j += NT) {
+            const uint32_t local = promo[j] & 0x3ffffffu, m = promo[j] >> 26;
+            atomicOr(&cnt[(size_t)m * y.wpc + (local >> kFshift)], kCmask << ((local & (kFpw - 1u)) * CBITS));
         }
     };
     auto stream_epoch = [&](bool undo) {
@@ -348,7 +379,7 @@ __global__ __launch_bounds__(NT, MINW) void traverse_block_kernel(QueryArgs a, B
 #pragma unroll
                 for (int e = 0; e < 8; e++) {
                     const int pos = pos0 + e;
-                    if (pos >= ra && pos < rb) visit(mcnt, (w[e >> 1] >> ((e & 1) * 16)) & 0xffffu, m, undo);
+                    if (pos >= ra && pos < rb) visit(mcnt, (w[e >> 1] >> ((e & 1) * 16)) & 0xffffu, undo);
                 }
             }
         }
@@ -368,23 +399,6 @@ __global__ __launch_bounds__(NT, MINW) void traverse_block_kernel(QueryArgs a, B
             }
         };
         auto process = [&](const uint4 (&r)[kUnroll], const int (&mr)[kUnroll]) {
-            if (undo) {
-#pragma unroll
-                for (int u = 0; u < kUnroll; u++) {
-                    if (mr[u] < 0) continue;
-                    uint32_t* mcnt = cnt + (size_t)mr[u] * y.wpc;
-                    const uint32_t w[4] = {r[u].x, r[u].y, r[u].z, r[u].w};
-#pragma unroll
-                    for (int e = 0; e < 8; e++) {
-                        const uint32_t local = (w[e >> 1] >> ((e & 1) * 16)) & 0xffffu;
-                        atomicSub(&mcnt[local >> kFshift], 1u << ((local & (kFpw - 1u)) * CBITS));
-                    }
-                }
-                return;
-            }
-            // all atomics of the batch first, then the (rare) promotions: a compare right
-            // behind each returning atomic would serialise on LDS latency
-            uint32_t old[kUnroll][8];
 #pragma unroll
             for (int u = 0; u < kUnroll; u++) {
                 if (mr[u] < 0) continue;
@@ -393,28 +407,24 @@ __global__ __launch_bounds__(NT, MINW) void traverse_block_kernel(QueryArgs a, B
 #pragma unroll
                 for (int e = 0; e < 8; e++) {
                     const uint32_t local = (w[e >> 1] >> ((e & 1) * 16)) & 0xffffu;
-                    old[u][e] = atomicAdd(&mcnt[local >> kFshift], 1u << ((local & (kFpw - 1u)) * CBITS));
-                }
-            }
-#pragma unroll
-            for (int u = 0; u < kUnroll; u++) {
-                if (mr[u] < 0) continue;
-                const uint32_t w[4] = {r[u].x, r[u].y, r[u].z, r[u].w};
-#pragma unroll
-                for (int e = 0; e < 8; e++) {
-                    const uint32_t local = (w[e >> 1] >> ((e & 1) * 16)) & 0xffffu;
-                    if (((old[u][e] >> ((local & (kFpw - 1u)) * CBITS)) & kCmask) == Lm1) {
-                        const uint32_t slot = atomicAdd(&misc[kPromoCount], 1u);
-                        if (slot < (uint32_t)kPromoCap) promo[slot] = local | ((uint32_t)mr[u] << 26);
-                    }
+                    const uint32_t one = 1u << ((local & (kFpw - 1u)) * CBITS);
+                    if (undo) atomicSub(&mcnt[local >> kFshift], one);
+                    else atomicAdd(&mcnt[local >> kFshift], one);
                 }
             }
         };
-        for (int g0 = 0; g0 < total; g0 += NT * kUnroll) {
-            uint4 r4[kUnroll];
-            int mr[kUnroll];
-            fetch(g0, r4, mr);
-            process(r4, mr);
+        // two register sets: the reads of one batch are in flight while the other is counted
+        uint4 r_a[kUnroll], r_b[kUnroll];
+        int m_a[kUnroll], m_b[kUnroll];
+        constexpr int kBatch = NT * kUnroll;
+        if (total > 0) fetch(0, r_a, m_a);
+        for (int g0 = 0; g0 < total; g0 += 2 * kBatch) {
+            if (g0 + kBatch < total) fetch(g0 + kBatch, r_b, m_b);
+            process(r_a, m_a);
+            if (g0 + kBatch < total) {
+                if (g0 + 2 * kBatch < total) fetch(g0 + 2 * kBatch, r_a, m_a);
+                process(r_b, m_b);
+            }
         }
         unsigned long long streamed = 0;
         for (int s = 0; s < S; s++) streamed += (unsigned long long)max(0, s_rb[s] - s_ra[s]);
@@ -426,7 +436,7 @@ __global__ __launch_bounds__(NT, MINW) void traverse_block_kernel(QueryArgs a, B
     int epoch = 0;
     for (; epoch < kMaxEpochs; epoch++) {
         // ---- 1. priority bound per composite ------------------------------------
-        if (tid < a.M) { s_rho[tid] = kInfBits; s_K[tid] = 0; s_active[tid] = 0; }
+        if (tid < a.M) { s_rho[tid] = kInfBits; s_K[tid] = 0; s_active[tid] = 0; s_hsum[tid] = 0.0f; }
         __syncthreads();
         if (tid < S) {
             const int c = s_c[tid], ns = s_ns[tid];
@@ -436,9 +446,23 @@ __global__ __launch_bounds__(NT, MINW) void traverse_block_kernel(QueryArgs a, B
                 const Stream st = load_stream(tid);
                 const int64_t jp = min((int64_t)c + s_stride[tid], (int64_t)ns) - 1;
                 probes++;
-                atomicMin(&s_rho[m], stream_prio_bits(st, (int)jp));
+                const uint32_t pi = stream_prio_bits(st, (int)jp);
+                atomicMin(&s_rho[m], pi);
                 atomicAdd(&s_active[m], 1u);
+                atomicAdd(&s_hsum[m], 1.0f / __builtin_bit_cast(float, pi));
             }
+        }
+        __syncthreads();
+        // The smallest of the streams' stride-end priorities lets only one stream use
+        // its whole stride and the epoch falls short of the steps it aimed at.  With
+        // windows locally equidistant in priority, the bound at which the streams
+        // together consume the sum of their strides is the harmonic mean of those
+        // priorities; any bound is valid, this one lands the epoch where intended.
+        // (A zero priority makes the mean 0 and a NaN makes it NaN: the minimum stays.)
+        if (tid < a.M && s_active[tid] > 0) {
+            const float hm = (float)s_active[tid] / s_hsum[tid];
+            if (hm > 0.0f && hm < __builtin_inff())
+                s_rho[tid] = max(s_rho[tid], __builtin_bit_cast(uint32_t, hm));
         }
         __syncthreads();
         phase(1);
@@ -475,6 +499,8 @@ __global__ __launch_bounds__(NT, MINW) void traverse_block_kernel(QueryArgs a, B
         // ---- 3. stream the new ranges ---------------------------------------------
         streamed += stream_epoch(false);
         __syncthreads();
+        collect_promotions();
+        __syncthreads();
         phase(3);
         const uint32_t np = misc[kPromoCount];
         // too many promotions at once (or no room left beside the ones still waiting
@@ -500,6 +526,8 @@ __global__ __launch_bounds__(NT, MINW) void traverse_block_kernel(QueryArgs a, B
                 continue;
             }
         }
+
+        mark_promotions(np);      // the epoch stands: later scans skip its promotions
 
         // ---- 4. exact step of every promotion -----------------------------------
         if (np > 0) {     // sample every stream's new range once; all rankings of the epoch share it
@@ -742,7 +770,9 @@ __global__ __launch_bounds__(NT, MINW) void traverse_block_kernel(QueryArgs a, B
                 const float t_armed = (float)(((unsigned long long)misc[kArmedHi] << 32) | misc[kArmedLo]);
                 k_target = fmaxf(t_armed + 1.0f, need) + (float)S;
             } else if (hint > 0.0f) {
-                k_target = (float)kmax < 0.9f * kHintFirst * hint ? kHintFirst * hint : kHintGrow * (float)kmax + (float)S;
+                const float so_far = (float)max(1u, misc[kNumCand] + misc[kEventCount]);   // promotions up to here
+                const float grow = fminf(kHintGrow, powf(1.0f + kPromoAim / so_far, inv_L));
+                k_target = (float)kmax < 0.9f * kHintFirst * hint ? kHintFirst * hint : grow * (float)kmax + (float)S;
             }
             k_target = fminf(k_target, 2.0f * (float)kmax + 16.0f * (float)S);
             if (shrunk) k_target = fminf(k_target, (float)kmax + (float)dk_lead);
@@ -825,7 +855,7 @@ bool block_traversal_supported(const QueryArgs& a, size_t* lds_bytes) {
     if (lds_bytes) *lds_bytes = y.lds_bytes;
     const int I = a.M * a.L;
     if (!a.inv || !a.lids || a.ppb > 65536) return false;
-    if (a.L > 255) return false;            // 4- and 8-bit visit counters only
+    if (a.L > 254) return false;            // 4- and 8-bit visit counters only
     if (4 * I > kBlockThreads || a.M > 64) return false;   // one thread per partial chunk of a stream
     if (a.kcap > 512) return false;
     if (a.ppb >= (1 << 25)) return false;
