@@ -90,19 +90,23 @@ __global__ void segsort_tile_kernel(const float* __restrict__ keys, SegGeom g,
 }
 
 // ---------------------------------------------------------------------------
-// LDS radix sort of one whole slice (4096 < points <= 32256) by one workgroup
-// (1024 threads up to 15360 points, 512 threads with more items each above:
-// the register file, not LDS, limits items per thread): least-significant-digit passes of 4 bits over the order-preserving
-// 32-bit image of the key.  Every thread owns IPT consecutive items in
-// registers (key + packed id/rank); a pass counts digits in per-thread private
-// 16-bit LDS counters laid out digit-major, scans the 16384 counters, and moves
-// keys, then ids, through one LDS staging buffer.  Thread-private counters plus
-// the digit-major scan make every pass stable, so equal keys keep ascending ids.
-// Nibbles that are constant over the slice (typically the exponent's) are
-// skipped.  Global traffic: keys read once, sorted keys / ids / inverse written
-// once, all coalesced.
+// LDS radix sort of one whole slice (512 < points <= 32256) by one workgroup:
+// least-significant-digit passes of 4 bits over the order-preserving 32-bit
+// image of the key.  Every thread owns IPT consecutive items in registers (key
+// + packed id/rank); a pass counts digits in per-thread private 16-bit LDS
+// counters laid out digit-major (with returning atomics, so that a thread's
+// updates pipeline), scans the 16 * threads counters, and moves keys, then ids,
+// through one LDS staging buffer.  Thread-private counters plus the digit-major
+// scan make every pass stable, so equal keys keep ascending ids.  Nibbles that
+// are constant over the slice (typically the exponent's) are skipped.  The
+// per-pass cost that does not depend on the slice (scan, barriers) grows with
+// the thread count, so the workgroup is the smallest of 64 / 128 / 256 / 512
+// threads that covers the slice with at most ~45 (512 threads: 63) items per
+// thread; a single wavefront needs no barrier at all.  Global traffic: keys
+// read once (all reads of a thread in flight together), sorted keys / ids /
+// inverse written once, all coalesced.
 constexpr int kRadixMax = 63 * 512;
-constexpr int kRadixMin = 4096;       // up to this the bitonic tile kernel is faster
+constexpr int kRadixMin = 512;        // up to this the bitonic tile kernel is faster
 
 template <int kRadixThreads, int IPT>
 __global__ __launch_bounds__(kRadixThreads) void segsort_radix_kernel(
@@ -125,10 +129,20 @@ __global__ __launch_bounds__(kRadixThreads) void segsort_radix_kernel(
     const int64_t base = i * g.n + off;
 
     if (tid < 2) misc[32 + tid] = tid ? 0xffffffffu : 0u;        // OR / AND of all keys
-    for (int j = tid; j < IPT * kRadixThreads; j += kRadixThreads)
-        stage[j] = j < n ? f2ord(keys[base + j] + 0.0f) : 0xffffffffu;   // pads sort last and stay last
-    __syncthreads();
     uint32_t k[IPT], rp[IPT];      // rp: id in the low half, rank / position in the high half
+    // coalesced reads, all in flight at once (the slice is read with one round trip),
+    // then through LDS into the blocked arrangement
+#pragma unroll
+    for (int r = 0; r < IPT; r++) {
+        const int j = min(r * kRadixThreads + tid, n - 1);       // unconditional: no branch per load
+        k[r] = __builtin_bit_cast(uint32_t, keys[base + j]);
+    }
+#pragma unroll
+    for (int r = 0; r < IPT; r++) {
+        const int j = r * kRadixThreads + tid;                    // pads sort last and stay last
+        stage[j] = j < n ? f2ord(__builtin_bit_cast(float, k[r]) + 0.0f) : 0xffffffffu;
+    }
+    __syncthreads();
     uint32_t vor = 0, vand = 0xffffffffu;
 #pragma unroll
     for (int r = 0; r < IPT; r++) {
@@ -153,13 +167,20 @@ __global__ __launch_bounds__(kRadixThreads) void segsort_radix_kernel(
 #pragma unroll
             for (int w = 0; w < 8; w++) cnt32[tid + w * kRadixThreads] = 0;
             __syncthreads();
+            // A returning atomic on the word that holds the counter (two neighbouring
+            // threads share a word): the LDS unit does the read-modify-write in issue
+            // order, so the IPT updates of a thread need no round trip between them.
+            const uint32_t half = (uint32_t)(tid & 1) * 16u;
+            uint32_t old[IPT];
 #pragma unroll
             for (int r = 0; r < IPT; r++) {
                 const uint32_t a = ((k[r] >> shift) & 15u) * kRadixThreads + tid;
-                const uint32_t c = cnt[a];
-                cnt[a] = (uint16_t)(c + 1);
-                rp[r] = (rp[r] & 0xffffu) | (c << 16);
+                old[r] = atomicAdd(&cnt32[a >> 1], 1u << half);
+                if ((r & 7) == 7) __builtin_amdgcn_sched_barrier(0);
             }
+#pragma unroll
+            for (int r = 0; r < IPT; r++)
+                rp[r] = (rp[r] & 0xffffu) | (((old[r] >> half) & 0xffffu) << 16);
         }
         __syncthreads();
         {   // exclusive scan of the 16*threads counters in memory order (digit-major)
@@ -210,14 +231,14 @@ __global__ __launch_bounds__(kRadixThreads) void segsort_radix_kernel(
         }
         __syncthreads();
 #pragma unroll
-        for (int r = 0; r < IPT; r++) {
-            stage16[rp[r] >> 16] = (uint16_t)rp[r];
+        for (int r = 0; r < IPT; r++) {      // ids move as whole words: 16-bit blocked reads would
+            stage[rp[r] >> 16] = rp[r] & 0xffffu;                // collide on LDS banks
             if ((r & 7) == 7) __builtin_amdgcn_sched_barrier(0);
         }
         __syncthreads();
 #pragma unroll
         for (int r = 0; r < IPT; r++) {
-            rp[r] = stage16[tid * IPT + r];
+            rp[r] = stage[tid * IPT + r];
             if ((r & 7) == 7) __builtin_amdgcn_sched_barrier(0);
         }
     }
@@ -365,8 +386,11 @@ int segsort(const float* d_keys, int num_indices, int64_t n, int block_size,
 #define DCIH_RADIX(NT, IPT) \
     if (g.ppb <= (int64_t)(NT) * (IPT))  \
         return launch_radix<NT, IPT>(d_keys, g, num_indices, d_skeys, d_sids, d_inv, d_lids, s)
-        DCIH_RADIX(1024, 3); DCIH_RADIX(1024, 7); DCIH_RADIX(1024, 11); DCIH_RADIX(1024, 15);
-        DCIH_RADIX(512, 37); DCIH_RADIX(512, 45); DCIH_RADIX(512, 53); DCIH_RADIX(512, 63);
+        DCIH_RADIX(64, 9); DCIH_RADIX(64, 17); DCIH_RADIX(64, 25); DCIH_RADIX(64, 33);
+        DCIH_RADIX(128, 21); DCIH_RADIX(128, 27); DCIH_RADIX(128, 33);
+        DCIH_RADIX(256, 21); DCIH_RADIX(256, 27); DCIH_RADIX(256, 33); DCIH_RADIX(256, 39); DCIH_RADIX(256, 45);
+        DCIH_RADIX(512, 27); DCIH_RADIX(512, 33); DCIH_RADIX(512, 39); DCIH_RADIX(512, 45);
+        DCIH_RADIX(512, 51); DCIH_RADIX(512, 57); DCIH_RADIX(512, 63);
 #undef DCIH_RADIX
     }
     if (g.tiles == 1) {
