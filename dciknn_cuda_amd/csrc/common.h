@@ -57,6 +57,53 @@ __device__ inline unsigned long long wave_max_u64(unsigned long long v) {
 }
 __device__ inline int lane_id() { return (int)(threadIdx.x & (kWave - 1)); }
 
+// Euclidean distances (compute_dist_device, src/dci_cuda_kernel.cu:36-44) from R
+// rows in global memory to the query held in LDS, by one wavefront.  With
+// 16-byte aligned rows (vec4) lane l sums the squares of elements 4l..4l+3,
+// 4l+256.., in ascending order, otherwise of elements l, l+64, ..; the lane sums
+// are then added across the wavefront.  Both traversal kernels call this, so a
+// point gets the same distance bits whichever kernel visits it; R > 1 only
+// interleaves the reads of independent rows.
+template <int R>
+__device__ inline void wave_row_dists(const float* const (&rows)[R], const float* q, int dim,
+                                      bool vec4, float (&dist)[R]) {
+    const int lane = lane_id();
+    float acc[R];
+#pragma unroll
+    for (int r = 0; r < R; r++) acc[r] = 0.f;
+    if (vec4) {
+        typedef float v4f __attribute__((ext_vector_type(4)));
+        for (int j = lane * 4; j < dim; j += kWave * 4) {
+            v4f x[R];
+#pragma unroll
+            for (int r = 0; r < R; r++) x[r] = *reinterpret_cast<const v4f*>(rows[r] + j);
+            const float q0 = q[j], q1 = q[j + 1], q2 = q[j + 2], q3 = q[j + 3];
+#pragma unroll
+            for (int r = 0; r < R; r++) {
+                float d = x[r].x - q0; acc[r] = __builtin_fmaf(d, d, acc[r]);
+                d = x[r].y - q1; acc[r] = __builtin_fmaf(d, d, acc[r]);
+                d = x[r].z - q2; acc[r] = __builtin_fmaf(d, d, acc[r]);
+                d = x[r].w - q3; acc[r] = __builtin_fmaf(d, d, acc[r]);
+            }
+        }
+    } else {
+        for (int j = lane; j < dim; j += kWave) {
+            const float qj = q[j];
+#pragma unroll
+            for (int r = 0; r < R; r++) {
+                const float d = rows[r][j] - qj;
+                acc[r] = __builtin_fmaf(d, d, acc[r]);
+            }
+        }
+    }
+#pragma unroll
+    for (int r = 0; r < R; r++) dist[r] = sqrtf(wave_sum(acc[r]));
+}
+// Whether every row of `data` starts on a 16-byte boundary.
+__device__ inline bool rows_vec4(const float* data, int dim) {
+    return (dim & 3) == 0 && (reinterpret_cast<uintptr_t>(data) & 15) == 0;
+}
+
 // In-place ascending bitonic sort of `n` (a power of two) 64-bit words in LDS
 // by all threads of the block.
 __device__ inline void bitonic_sort_u64(unsigned long long* s, int n) {

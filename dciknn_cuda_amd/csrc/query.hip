@@ -201,13 +201,10 @@ __global__ __launch_bounds__(kWave) void traverse_kernel(QueryArgs a, Layout y) 
                         pm &= pm - 1;
                         const int cpt = __shfl(pt, src, kWave);
                         // exact distance (:36-44), row read by the whole wavefront
-                        const float* row = a.data + (int64_t)cpt * a.dim;
-                        float acc = 0.f;
-                        for (int j = lane; j < a.dim; j += kWave) {
-                            const float df = row[j] - s_q[j];
-                            acc = __builtin_fmaf(df, df, acc);
-                        }
-                        const float dist = sqrtf(wave_sum(acc));
+                        const float* const rows1[1] = {a.data + (int64_t)cpt * a.dim};
+                        float dist1[1];
+                        wave_row_dists<1>(rows1, s_q, a.dim, rows_vec4(a.data, a.dim), dist1);
+                        const float dist = dist1[0];
                         const unsigned long long e =
                             ((unsigned long long)__builtin_bit_cast(uint32_t, dist) << 32) | (uint32_t)cpt;
                         ncand++;

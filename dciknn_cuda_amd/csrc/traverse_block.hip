@@ -38,8 +38,6 @@ namespace dcih {
 
 namespace {
 
-constexpr int kPromoCap = 256;      // promotions one epoch may produce
-constexpr int kPromoMax = 160;       // above this an epoch is undone and halved
 constexpr int kMaxEpochs = 100000;
 constexpr uint32_t kInfBits = 0x7f800000u;
 
@@ -57,6 +55,8 @@ struct BlockLayout {
     int off_q;        // query row
     int off_samp;     // per stream: 16 sampled window priorities of the current epoch's range
     int off_promo, off_events, off_acc, off_sort, off_cnt;
+    int promo_cap;    // promotions one epoch may produce (table size)
+    int promo_max;    // above this an epoch is undone and halved
     int event_cap;    // promotions waiting for the other composites (= accepted candidates per replay)
     int sort_cap;     // power of two >= kcap + 128: top-k plus one batch of candidates
     size_t lds_bytes;
@@ -84,11 +84,16 @@ BlockLayout make_block_layout(const QueryArgs& a) {
     y.off_q = o;        o += ((a.dim + 3) & ~3) * 4;
     // small tables keep more workgroups resident per CU; an item that overflows them
     // is redone by the step-by-step kernel
-    y.event_cap = 512;
+    // The tables grow with the promotions a stop needs (about k * T, more when the
+    // step limit rather than c0 >= k ends the traversal): fewer, larger epochs.
+    y.promo_cap = 256;
+    while (y.promo_cap < 2 * (int64_t)a.k * a.T && y.promo_cap < 2048) y.promo_cap <<= 1;
+    y.promo_max = y.promo_cap * 5 / 8;
+    y.event_cap = 2 * y.promo_cap;
     y.sort_cap = 256;          // top-k plus a batch of at least 128 new candidates
     while (y.sort_cap < a.kcap + 128) y.sort_cap <<= 1;
     y.off_samp = o;     o += 2 * I * 16 * 4;
-    y.off_promo = o;    o += kPromoCap * 4;
+    y.off_promo = o;    o += y.promo_cap * 4;
     y.off_acc = o;      o += y.event_cap * 4;
     o = (o + 15) & ~15;
     y.off_events = o;   o += y.event_cap * 8;
@@ -249,14 +254,17 @@ __global__ __launch_bounds__(NT, MINW) void traverse_block_kernel(QueryArgs a, B
     // high power (L) of the steps taken, so stop steps of one partition scatter
     // little and most items finish in one or two epochs, while a jump 20 % too far
     // already brings several times the promotions needed and overflows the tables.
-    // Where the stop needs more promotions than one epoch may produce (about
-    // k * T, against kPromoMax), the jump is shortened by the same power law so
-    // that an epoch yields about 0.6 * kPromoMax of them.
-    constexpr float kHintGrow = 1.06f, kPromoAim = 0.6f * (float)kPromoMax;
+    // Where the stop needs more promotions than one epoch may produce (their
+    // number at earlier stops in this partition is the second hint; about k * T
+    // without one), the jump is shortened by the same power law so that an epoch
+    // yields about 0.6 * promo_max of them.
+    constexpr float kHintGrow = 1.06f;
+    const float kPromoAim = 0.6f * (float)y.promo_max;
     const float inv_L = 1.0f / (float)a.L;
-    const float kHintFirst =
-        fminf(1.05f, powf(kPromoAim / fmaxf(1.0f, (float)a.k * (float)T), inv_L));
     const float hint = a.stop_hint ? a.stop_hint[b] : 0.0f;
+    const float hint_promos = a.stop_hint ? a.stop_hint[a.B + b] : 0.0f;
+    const float kHintFirst = fminf(1.05f,
+        powf(kPromoAim / fmaxf(1.0f, hint_promos > 0.0f ? hint_promos : (float)a.k * (float)T), inv_L));
     {
         int first = 4;
         for (int s = 0; s < S; s++) first = max(first, s_ns[s] / 128);
@@ -327,7 +335,7 @@ __global__ __launch_bounds__(NT, MINW) void traverse_block_kernel(QueryArgs a, B
             for (uint32_t f = 0; f < kFpw; f++) {
                 if (((x >> (f * CBITS)) & kCmask) == 0u) {
                     const uint32_t slot = atomicAdd(&misc[kPromoCount], 1u);
-                    if (slot < (uint32_t)kPromoCap) promo[slot] = (first + f) | ((uint32_t)m << 26);
+                    if (slot < (uint32_t)y.promo_cap) promo[slot] = (first + f) | ((uint32_t)m << 26);
                 }
             }
         }
@@ -432,7 +440,8 @@ __global__ __launch_bounds__(NT, MINW) void traverse_block_kernel(QueryArgs a, B
     };
 
     unsigned long long streamed = 0;     // entries streamed so far (same on every thread)
-    bool shrunk = false;
+    bool shrunk = false;        // the previous epoch was undone
+    bool undone_once = false;   // some epoch of this item was undone
     int epoch = 0;
     for (; epoch < kMaxEpochs; epoch++) {
         // ---- 1. priority bound per composite ------------------------------------
@@ -459,7 +468,9 @@ __global__ __launch_bounds__(NT, MINW) void traverse_block_kernel(QueryArgs a, B
         // together consume the sum of their strides is the harmonic mean of those
         // priorities; any bound is valid, this one lands the epoch where intended.
         // (A zero priority makes the mean 0 and a NaN makes it NaN: the minimum stays.)
-        if (tid < a.M && s_active[tid] > 0) {
+        // Once an epoch had to be undone the smallest priority is kept: then no stream
+        // passes its stride, and halving the strides is sure to shrink the epoch.
+        if (!undone_once && tid < a.M && s_active[tid] > 0) {
             const float hm = (float)s_active[tid] / s_hsum[tid];
             if (hm > 0.0f && hm < __builtin_inff())
                 s_rho[tid] = max(s_rho[tid], __builtin_bit_cast(uint32_t, hm));
@@ -505,10 +516,10 @@ __global__ __launch_bounds__(NT, MINW) void traverse_block_kernel(QueryArgs a, B
         const uint32_t np = misc[kPromoCount];
         // too many promotions at once (or no room left beside the ones still waiting
         // for the other composites): take the epoch back and retry with half the stride
-        if (np > (uint32_t)kPromoMax || misc[kEventCount] + np > (uint32_t)y.event_cap) {
+        if (np > (uint32_t)y.promo_max || misc[kEventCount] + np > (uint32_t)y.event_cap) {
             bool minimal = true;
             for (int s2 = 0; s2 < S; s2++) minimal = minimal && s_stride[s2] <= 1;
-            if (minimal && np <= (uint32_t)kPromoCap && misc[kEventCount] + np <= (uint32_t)y.event_cap) {
+            if (minimal && np <= (uint32_t)y.promo_cap && misc[kEventCount] + np <= (uint32_t)y.event_cap) {
                 // cannot go smaller; the tables still hold it
             } else if (minimal) {
                 if (tid == 0) misc[kFail] = 2;
@@ -521,6 +532,7 @@ __global__ __launch_bounds__(NT, MINW) void traverse_block_kernel(QueryArgs a, B
                 if (tid < S) s_stride[tid] = max(1, s_stride[tid] / 2);
                 if (tid == 0) misc[kPromoCount] = 0;
                 shrunk = true;
+                undone_once = true;
                 __syncthreads();
                 phase(4);
                 continue;
@@ -729,17 +741,20 @@ __global__ __launch_bounds__(NT, MINW) void traverse_block_kernel(QueryArgs a, B
         for (int done = 0; done < nacc;) {      // in batches that fit beside the top-k
             const int topn = (int)misc[kTopN];
             const int batch = min(nacc - done, y.sort_cap - topn);
-            for (int c = wave; c < batch; c += kWaves) {
-                const int64_t pt = off + acc[done + c];
-                const float* row = a.data + pt * a.dim;
-                float sum = 0.f;
-                for (int j = lane; j < a.dim; j += kWave) {
-                    const float df = row[j] - s_q[j];
-                    sum = __builtin_fmaf(df, df, sum);
+            // two candidates per wavefront at a time: their row reads overlap
+            const bool vec4 = rows_vec4(a.data, a.dim);
+            for (int c = wave; c < batch; c += 2 * kWaves) {
+                const int c2 = c + kWaves;
+                const int64_t pt0 = off + acc[done + c];
+                const int64_t pt1 = c2 < batch ? off + acc[done + c2] : pt0;
+                const float* const rows2[2] = {a.data + pt0 * a.dim, a.data + pt1 * a.dim};
+                float d2[2];
+                wave_row_dists<2>(rows2, s_q, a.dim, vec4, d2);
+                if (lane == 0) {
+                    sortbuf[topn + c] = ((unsigned long long)__builtin_bit_cast(uint32_t, d2[0]) << 32) | (uint32_t)pt0;
+                    if (c2 < batch)
+                        sortbuf[topn + c2] = ((unsigned long long)__builtin_bit_cast(uint32_t, d2[1]) << 32) | (uint32_t)pt1;
                 }
-                const float dist = sqrtf(wave_sum(sum));
-                if (lane == 0)
-                    sortbuf[topn + c] = ((unsigned long long)__builtin_bit_cast(uint32_t, dist) << 32) | (uint32_t)pt;
             }
             int np2 = 2;
             while (np2 < topn + batch) np2 <<= 1;
@@ -775,7 +790,8 @@ __global__ __launch_bounds__(NT, MINW) void traverse_block_kernel(QueryArgs a, B
                 k_target = (float)kmax < 0.9f * kHintFirst * hint ? kHintFirst * hint : grow * (float)kmax + (float)S;
             }
             k_target = fminf(k_target, 2.0f * (float)kmax + 16.0f * (float)S);
-            if (shrunk) k_target = fminf(k_target, (float)kmax + (float)dk_lead);
+            if (shrunk) k_target = fminf(k_target, (float)kmax + 2.0f * (float)dk_lead);
+            shrunk = false;       // the epoch after an undo was accepted: back to aimed epochs
             __syncthreads();
             if (tid < S) {
                 const int m = (tid >> 1) / a.L;
@@ -813,6 +829,9 @@ __global__ __launch_bounds__(NT, MINW) void traverse_block_kernel(QueryArgs a, B
         const float cur = (float)((((unsigned long long)misc[kStopStepHi] << 32) | misc[kStopStepLo]) + 1);
         const float old = a.stop_hint[b];     // racy on purpose: any recent value will do
         a.stop_hint[b] = old > 0.0f ? 0.75f * old + 0.25f * cur : cur;
+        const float curp = (float)(misc[kNumCand] + misc[kEventCount]);
+        const float oldp = a.stop_hint[a.B + b];
+        a.stop_hint[a.B + b] = oldp > 0.0f ? 0.75f * oldp + 0.25f * curp : curp;
     }
     // ---- results -------------------------------------------------------------------
     const int topn = (int)misc[kTopN];
