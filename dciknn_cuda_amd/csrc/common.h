@@ -105,8 +105,26 @@ __device__ inline bool rows_vec4(const float* data, int dim) {
 }
 
 // In-place ascending bitonic sort of `n` (a power of two) 64-bit words in LDS
-// by all threads of the block.
+// by all threads of the block (which has at least one full wavefront).
 __device__ inline void bitonic_sort_u64(unsigned long long* s, int n) {
+    if (n <= kWave) {
+        // one wavefront sorts in registers with lane exchanges: no barrier per stage
+        __syncthreads();
+        if (threadIdx.x < kWave) {
+            const int lane = (int)threadIdx.x;
+            unsigned long long v = lane < n ? s[lane] : ~0ull;
+            for (int size = 2; size <= n; size <<= 1) {
+                for (int stride = size >> 1; stride > 0; stride >>= 1) {
+                    const unsigned long long o = __shfl_xor(v, stride, kWave);
+                    const bool keep_min = ((lane & stride) == 0) == ((lane & size) == 0);
+                    v = keep_min ? (v < o ? v : o) : (v > o ? v : o);
+                }
+            }
+            if (lane < n) s[lane] = v;
+        }
+        __syncthreads();
+        return;
+    }
     for (int size = 2; size <= n; size <<= 1) {
         for (int stride = size >> 1; stride > 0; stride >>= 1) {
             __syncthreads();
