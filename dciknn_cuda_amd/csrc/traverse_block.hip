@@ -47,7 +47,7 @@ enum Misc {   // 32-bit scalars shared by the workgroup; kStreamedLo must stay 8
 };
 
 struct BlockLayout {
-    int cbits, wpc, seen_words, counter_words;
+    int cbits, wpc, seen_words, mark_words, counter_words;
     int off_idx;      // per simple index: p, qp            (2 * I words)
     int off_stream;   // per stream: consumed, previous, total, range lo/hi, chunks, pos0, prefix (10 * 2I + 1 words, incl. stride and composite number)
     int off_chunk0;   // per stream: global index of its first 16-byte chunk (2I 64-bit words)
@@ -63,8 +63,7 @@ struct BlockLayout {
 };
 
 __host__ __device__ inline int counter_bits_of(int L) {
-    // the all-ones value of a field marks a point already promoted, so L stays below it
-    return L <= 14 ? 4 : (L <= 254 ? 8 : (L <= 65534 ? 16 : 32));
+    return L <= 15 ? 4 : (L <= 255 ? 8 : (L <= 65535 ? 16 : 32));
 }
 
 BlockLayout make_block_layout(const QueryArgs& a) {
@@ -74,7 +73,10 @@ BlockLayout make_block_layout(const QueryArgs& a) {
     const int64_t fpw = 32 / y.cbits;
     y.wpc = (int)((a.ppb + fpw - 1) / fpw);
     y.seen_words = (int)((a.ppb + 31) / 32);
-    y.counter_words = a.M * y.wpc + y.seen_words;
+    // promoted points are marked by the all-ones counter value; where L itself is that
+    // value (15, 255) a bitmap per composite marks them instead
+    y.mark_words = a.L == (1 << y.cbits) - 1 ? a.M * y.seen_words : 0;
+    y.counter_words = a.M * y.wpc + y.seen_words + y.mark_words;
     int o = kMiscWords * 4;
     y.off_idx = o;      o += 2 * I * 4;
     y.off_stream = o;   o += (10 * 2 * I + 2) * 4;
@@ -189,6 +191,7 @@ __global__ __launch_bounds__(NT, MINW) void traverse_block_kernel(QueryArgs a, B
     unsigned long long* sortbuf = reinterpret_cast<unsigned long long*>(smem + y.off_sort);
     uint32_t* cnt = reinterpret_cast<uint32_t*>(smem + y.off_cnt);
     uint32_t* seen = cnt + (size_t)a.M * y.wpc;
+    uint32_t* marked = seen + y.seen_words;          // only where y.mark_words > 0
 
     const int tid = threadIdx.x;
     const int lane = tid & (kWave - 1);
@@ -320,8 +323,8 @@ __global__ __launch_bounds__(NT, MINW) void traverse_block_kernel(QueryArgs a, B
     };
     // Counters that stand at exactly L belong to points promoted in this epoch:
     // a point is visited once per simple index, so its counter never passes L, and
-    // promotions of earlier epochs were moved to the all-ones value when their
-    // epoch was accepted (mark_promotions).
+    // promotions of earlier epochs were moved to the all-ones value (or, where L is
+    // that value, entered in a bitmap) when their epoch was accepted (mark_promotions).
     auto collect_promotions = [&]() {
         constexpr uint32_t kRep = CBITS == 4 ? 0x11111111u : 0x01010101u;
         const uint32_t want = (uint32_t)a.L * kRep;
@@ -334,6 +337,8 @@ __global__ __launch_bounds__(NT, MINW) void traverse_block_kernel(QueryArgs a, B
 #pragma unroll
             for (uint32_t f = 0; f < kFpw; f++) {
                 if (((x >> (f * CBITS)) & kCmask) == 0u) {
+                    if (y.mark_words > 0 &&
+                        ((marked[m * y.seen_words + ((first + f) >> 5)] >> ((first + f) & 31u)) & 1u)) continue;
                     const uint32_t slot = atomicAdd(&misc[kPromoCount], 1u);
                     if (slot < (uint32_t)y.promo_cap) promo[slot] = (first + f) | ((uint32_t)m << 26);
                 }
@@ -343,7 +348,8 @@ __global__ __launch_bounds__(NT, MINW) void traverse_block_kernel(QueryArgs a, B
     auto mark_promotions = [&](uint32_t np) {
         for (uint32_t j = tid; j < np; j += NT) {
             const uint32_t local = promo[j] & 0x3ffffffu, m = promo[j] >> 26;
-            atomicOr(&cnt[(size_t)m * y.wpc + (local >> kFshift)], kCmask << ((local & (kFpw - 1u)) * CBITS));
+            if (y.mark_words > 0) atomicOr(&marked[m * y.seen_words + (local >> 5)], 1u << (local & 31u));
+            else atomicOr(&cnt[(size_t)m * y.wpc + (local >> kFshift)], kCmask << ((local & (kFpw - 1u)) * CBITS));
         }
     };
     auto stream_epoch = [&](bool undo) {
@@ -874,7 +880,7 @@ bool block_traversal_supported(const QueryArgs& a, size_t* lds_bytes) {
     if (lds_bytes) *lds_bytes = y.lds_bytes;
     const int I = a.M * a.L;
     if (!a.inv || !a.lids || a.ppb > 65536) return false;
-    if (a.L > 254) return false;            // 4- and 8-bit visit counters only
+    if (a.L > 255) return false;            // 4- and 8-bit visit counters only
     if (4 * I > kBlockThreads || a.M > 64) return false;   // one thread per partial chunk of a stream
     if (a.kcap > 512) return false;
     if (a.ppb >= (1 << 25)) return false;
