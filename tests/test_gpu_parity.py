@@ -158,6 +158,9 @@ CASES = [
     (257, 16, 12, 2, 20, 3, 5, 257, 10, "normal"),          # k = n, 8-bit counters
     (4000, 16, 24, 2, 10, 2, 16, 100, 30, "grid"),          # ties everywhere
     (1500, 8, 10, 70, 1, 6, 8, 4, 15, "normal"),            # more than 64 simple indices
+    (40000, 16, 24, 2, 12, 2, 16, 10, 200, "normal"),       # step limit ends it: hundreds of promotions, large tables
+    (30000, 16, 16, 2, 15, 2, 4, 50, 300, "normal"),        # L = 15: 4-bit counters with the promoted bitmap
+    (30000, 16, 16, 2, 14, 3, 8, 40, 100, "normal"),        # L = 14: promoted points marked in the counters
 ]
 
 
