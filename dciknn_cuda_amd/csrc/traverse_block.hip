@@ -156,6 +156,39 @@ __device__ inline unsigned long long pack_event(uint32_t time, int m, bool lane0
            ((unsigned long long)(lane0 ? 1u : 0u) << 25) | local;
 }
 
+// Partition point of a monotone predicate (true, then false) over [lo, hi), found by
+// a group of G = 2^lg consecutive lanes that probe the midpoints of G equal parts per
+// round: log_G rounds of dependent reads instead of log_2.  A group lies within one
+// wavefront and starts at lane `gbase`; `g` is the lane's place in it.  Every lane of
+// the wavefront must call this (the rounds are wave-uniform); lanes without a group
+// pass active = false.  hi - lo must stay below 2^31 / (2 G).
+template <class Pred>
+__device__ inline int group_partition_point(int lo, int hi, bool active, int lg, int gbase, int g,
+                                            Pred pred, uint32_t& probes) {
+    const int G = 1 << lg;
+    if (!active) { lo = 0; hi = 0; }
+    while (__any(lo < hi)) {
+        const bool busy = lo < hi;
+        const uint32_t len = (uint32_t)(hi - lo);
+        bool t = false;
+        if (busy) {
+            probes++;
+            t = pred(lo + (int)((len * (uint32_t)(2 * g + 1)) >> (lg + 1)));
+        }
+        const unsigned long long m = __ballot(t);
+        if (busy) {
+            // positions rise with the lane and the predicate is monotone: the hits are a prefix
+            const int hits = __popcll((m >> gbase) & ((1ull << G) - 1ull));
+            const int last_hit = lo + (int)((len * (uint32_t)(2 * hits - 1)) >> (lg + 1));     // lane hits-1
+            const int first_miss = lo + (int)((len * (uint32_t)(2 * hits + 1)) >> (lg + 1));   // lane hits
+            if (hits < G) hi = first_miss;
+            if (hits > 0) lo = last_hit + 1;
+        }
+    }
+    return lo;
+}
+__host__ __device__ inline int floor_log2(int v) { int l = 0; while ((2 << l) <= v) l++; return l; }
+
 // MINW = waves per SIMD the register allocation must leave room for: LDS decides how
 // many workgroups fit a CU, and the kernel should not be the tighter limit.
 template <int NT, int CBITS, int MINW>
@@ -227,22 +260,24 @@ __global__ __launch_bounds__(NT, MINW) void traverse_block_kernel(QueryArgs a, B
     for (int j = tid; j < a.dim; j += NT) s_q[j] = a.query[(int64_t)qi * a.dim + j];
     if (tid < kMiscWords) misc[tid] = 0;
     uint32_t probes = 0;
-    if (tid < I) {      // positioning search (:279-297)
-        const float* key = a.skeys + (int64_t)tid * a.N + off;
-        const float qp = a.qproj[(int64_t)tid * a.nq + qi];
-        int lo = 0, hi = n;    // first position whose key is not below qp
-        while (lo < hi) {
-            const int mid = (lo + hi) >> 1;
-            probes++;
-            if (key[mid] < qp) lo = mid + 1; else hi = mid;
-        }
-        const int p = lo - 1;
-        s_p[tid] = p;
-        s_qp[tid] = qp;
-        for (int side = 0; side < 2; side++) {
-            s_ns[2 * tid + side] = stream_windows(n, T, p, side);
-            s_c[2 * tid + side] = 0;
-            s_mof[2 * tid + side] = tid / a.L;
+    {   // positioning search (:279-297): first position whose key is not below qp,
+        // one group of lanes per simple index
+        const int lg = min(3, floor_log2(kWave / ((I + kWaves - 1) / kWaves))), G = 1 << lg;
+        const int slot = lane >> lg, i = wave * (kWave >> lg) + slot;
+        const bool active = i < I;
+        const float* key = a.skeys + (int64_t)(active ? i : 0) * a.N + off;
+        const float qp = active ? a.qproj[(int64_t)i * a.nq + qi] : 0.f;
+        const int lo = group_partition_point(0, n, active, lg, slot * G, lane - slot * G,
+                                             [&](int j) { return key[j] < qp; }, probes);
+        if (active && lane == slot * G) {
+            const int p = lo - 1;
+            s_p[i] = p;
+            s_qp[i] = qp;
+            for (int side = 0; side < 2; side++) {
+                s_ns[2 * i + side] = stream_windows(n, T, p, side);
+                s_c[2 * i + side] = 0;
+                s_mof[2 * i + side] = i / a.L;
+            }
         }
     }
     __syncthreads();
@@ -484,28 +519,34 @@ __global__ __launch_bounds__(NT, MINW) void traverse_block_kernel(QueryArgs a, B
         __syncthreads();
         phase(1);
         // ---- 2. how far each stream goes: all windows with priority <= bound ----
-        if (tid < S) {
-            const int c = s_c[tid], ns = s_ns[tid];
-            const int m = (tid >> 1) / a.L;
+        {   // one group of lanes per stream; search window by window (twice the stride,
+            // then four times as much, ...) so that probes stay near what will be streamed
+            const int lg = min(3, floor_log2(kWave / ((S + kWaves - 1) / kWaves))), G = 1 << lg;
+            const int slot = lane >> lg, sidx = wave * (kWave >> lg) + slot, g = lane - slot * G;
+            const bool active = sidx < S;
+            const int c = active ? s_c[sidx] : 0, ns = active ? s_ns[sidx] : 0;
+            const int m = active ? (sidx >> 1) / a.L : 0;
             const uint32_t rho = s_rho[m];
-            int cn = c;
-            if (c < ns && rho < kInfBits) {
-                const Stream st = load_stream(tid);
-                // gallop to an upper bound, then bisect
-                int64_t step = s_stride[tid];
-                int lo = c, hi = (int)min((int64_t)ns, (int64_t)c + step);
-                while (hi < ns) {
-                    probes++;
-                    if (stream_prio_bits(st, hi - 1) <= rho) {
-                        lo = hi; step *= 2; hi = (int)min((int64_t)ns, (int64_t)hi + step);
-                    } else break;
+            const Stream st = load_stream(active ? sidx : 0);
+            bool more = active && c < ns && rho < kInfBits;
+            const bool searched = more;
+            int lo = c, hi = c;
+            int64_t span = 2 * (int64_t)(active ? s_stride[sidx] : 1);
+            while (__any(more)) {
+                if (more) hi = (int)min((int64_t)ns, (int64_t)lo + span);
+                const int r = group_partition_point(lo, hi, more, lg, slot * G, g,
+                    [&](int j) { return stream_prio_bits(st, j) <= rho; }, probes);
+                if (more) {
+                    if (r == hi && hi < ns) { lo = hi; span *= 4; }
+                    else { lo = r; more = false; }
                 }
-                cn = count_below(st, rho, false, lo, hi, probes);
-            } else if (c < ns) {
-                cn = ns;     // NaN priorities: take the rest so the epoch loop ends
             }
-            s_c[tid] = cn;
-            atomicAdd(&s_K[m], (uint32_t)cn);
+            // (NaN priorities: take the rest so the epoch loop ends)
+            const int cn = searched ? lo : (active && c < ns ? ns : c);
+            if (active && g == 0) {
+                s_c[sidx] = cn;
+                atomicAdd(&s_K[m], (uint32_t)cn);
+            }
         }
         __syncthreads();
         bool all_done = true;
