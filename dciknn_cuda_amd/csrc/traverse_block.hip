@@ -92,11 +92,14 @@ BlockLayout make_block_layout(const QueryArgs& a) {
     while (y.promo_cap < 2 * (int64_t)a.k * a.T && y.promo_cap < 2048) y.promo_cap <<= 1;
     y.promo_max = y.promo_cap * 5 / 8;
     y.event_cap = 2 * y.promo_cap;
-    y.sort_cap = 256;          // top-k plus a batch of at least 128 new candidates
-    while (y.sort_cap < a.kcap + 128) y.sort_cap <<= 1;
-    y.off_samp = o;     o += 2 * I * 16 * 4;
-    y.off_promo = o;    o += y.promo_cap * 4;
-    y.off_acc = o;      o += y.event_cap * 4;
+    y.sort_cap = 64;           // top-k plus a batch of at least 48 new candidates
+    while (y.sort_cap < a.kcap + 48) y.sort_cap <<= 1;
+    // the accepted candidates of a replay share the room of the priority samples and the
+    // promotion list, both of which the ranking before it has finished with
+    y.off_samp = o;
+    y.off_acc = o;
+    o += max(2 * I * 16 * 4 + y.promo_cap * 4, y.event_cap * 4);
+    y.off_promo = y.off_samp + 2 * I * 16 * 4;
     o = (o + 15) & ~15;
     y.off_events = o;   o += y.event_cap * 8;
     y.off_sort = o;     o += y.sort_cap * 8;
@@ -934,7 +937,7 @@ bool block_traversal_supported(const QueryArgs& a, size_t* lds_bytes) {
 int query_block(const QueryArgs& a, hipStream_t s) {
     const BlockLayout y = make_block_layout(a);
     const int64_t items = (int64_t)a.nq * a.B;
-    const bool many = 160 * 1024 / y.lds_bytes >= 4;     // four or more workgroups per CU by LDS
+    const int fit = (int)(160 * 1024 / y.lds_bytes);      // workgroups per CU by LDS
 #define DCIH_LAUNCH(CB, MW)                                                                        \
     do {                                                                                           \
         static bool attr_done = false;                                                             \
@@ -946,8 +949,8 @@ int query_block(const QueryArgs& a, hipStream_t s) {
         hipLaunchKernelGGL((traverse_block_kernel<kBlockThreads, CB, MW>), dim3((unsigned)items),  \
                            dim3(kBlockThreads), y.lds_bytes, s, a, y);                             \
     } while (0)
-    if (y.cbits == 4) { if (many) DCIH_LAUNCH(4, 4); else DCIH_LAUNCH(4, 3); }
-    else              { if (many) DCIH_LAUNCH(8, 4); else DCIH_LAUNCH(8, 3); }
+    if (y.cbits == 4) { if (fit >= 6) DCIH_LAUNCH(4, 6); else if (fit >= 5) DCIH_LAUNCH(4, 5); else if (fit == 4) DCIH_LAUNCH(4, 4); else DCIH_LAUNCH(4, 3); }
+    else              { if (fit >= 6) DCIH_LAUNCH(8, 6); else if (fit >= 5) DCIH_LAUNCH(8, 5); else if (fit == 4) DCIH_LAUNCH(8, 4); else DCIH_LAUNCH(8, 3); }
 #undef DCIH_LAUNCH
     DCIH_HIP(hipGetLastError());
     return 0;
