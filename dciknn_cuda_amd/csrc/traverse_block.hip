@@ -39,6 +39,7 @@ namespace dcih {
 namespace {
 
 constexpr int kMaxEpochs = 100000;
+constexpr int kXcds = 8;             // accelerator dies of an MI355X, each with its own L2
 constexpr uint32_t kInfBits = 0x7f800000u;
 
 enum Misc {   // 32-bit scalars shared by the workgroup; kStreamedLo must stay 8-byte aligned
@@ -246,9 +247,17 @@ __global__ __launch_bounds__(NT, MINW) void traverse_block_kernel(QueryArgs a, B
     const int S = 2 * I;                       // streams
     const uint32_t Lm1 = (uint32_t)a.L - 1u;
 
-    const int64_t item = blockIdx.x;
-    const int b = (int)(item % a.B);
-    const int qi = (int)(item / a.B);
+    // Workgroups go to the XCDs round-robin by their number, and every XCD has an L2
+    // of its own.  XCD x gets the partitions x, x + 8, ... and works through them one
+    // after the other, all queries of a partition before the next: the workgroups an
+    // XCD runs at any moment share one partition's slices (a few MB), which then live
+    // in that L2 instead of being fetched again by every query.
+    const int xcd = (int)(blockIdx.x % kXcds);
+    const int64_t seq = blockIdx.x / kXcds;
+    const int b = xcd + kXcds * (int)(seq / a.nq);
+    const int qi = (int)(seq % a.nq);
+    if (b >= a.B) return;                      // this XCD has one partition fewer than others
+    const int64_t item = (int64_t)qi * a.B + b;
     const int64_t off = (int64_t)b * a.ppb;
     const int n = (int)min(a.N - off, a.ppb);
     unsigned long long* part_out = a.part + item * a.kcap;
@@ -930,13 +939,13 @@ bool block_traversal_supported(const QueryArgs& a, size_t* lds_bytes) {
     if (a.ppb >= (1 << 25)) return false;
     if ((int64_t)a.L * (a.ppb + 2 * (int64_t)a.T) >= 0x7fffffffLL) return false;   // steps fit 32 bits
     if ((int64_t)a.ppb + 2 * (int64_t)a.T >= 0x7fffffffLL) return false;
-    if ((int64_t)a.nq * a.B > 0x7fffffffLL) return false;
+    if ((int64_t)a.nq * (a.B + kXcds) > 0x7fffffffLL) return false;
     return y.lds_bytes <= 160 * 1024 - 512;
 }
 
 int query_block(const QueryArgs& a, hipStream_t s) {
     const BlockLayout y = make_block_layout(a);
-    const int64_t items = (int64_t)a.nq * a.B;
+    const int64_t items = (int64_t)a.nq * kXcds * ((a.B + kXcds - 1) / kXcds);
     const int fit = (int)(160 * 1024 / y.lds_bytes);      // workgroups per CU by LDS
 #define DCIH_LAUNCH(CB, MW)                                                                        \
     do {                                                                                           \
