@@ -446,18 +446,33 @@ __global__ __launch_bounds__(NT, MINW) void traverse_block_kernel(QueryArgs a, B
         }
         // whole chunks
         const int total = s_pref[S];
-        int cur = 0;
+        // The stream a thread is in changes rarely: its description stays in registers and
+        // LDS is read only when a chunk number passes the end of the stream.  Addresses of
+        // a batch are all formed before its reads are issued, and the reads themselves are
+        // unconditional (a thread past the end re-reads the first chunk and ignores it), so
+        // they go out back to back.
+        int cur = 0, next_pref = s_pref[1], mof = s_mof[0];
+        long long delta = s_chunk0[0] + 1 - s_pref[0];      // chunk number -> index into `all`
         auto fetch = [&](int g0, uint4 (&r)[kUnroll], int (&mr)[kUnroll]) {
+            const uint4* ptr[kUnroll];
 #pragma unroll
             for (int u = 0; u < kUnroll; u++) {
                 const int g = g0 + u * NT + tid;
                 mr[u] = -1;
+                ptr[u] = all;
                 if (g < total) {
-                    while (g >= s_pref[cur + 1]) cur++;
-                    mr[u] = s_mof[cur];
-                    r[u] = all[s_chunk0[cur] + 1 + (g - s_pref[cur])];
+                    while (g >= next_pref) {
+                        cur++;
+                        next_pref = s_pref[cur + 1];
+                        mof = s_mof[cur];
+                        delta = s_chunk0[cur] + 1 - s_pref[cur];
+                    }
+                    mr[u] = mof;
+                    ptr[u] = all + (delta + g);
                 }
             }
+#pragma unroll
+            for (int u = 0; u < kUnroll; u++) r[u] = *ptr[u];
         };
         auto process = [&](const uint4 (&r)[kUnroll], const int (&mr)[kUnroll]) {
 #pragma unroll
