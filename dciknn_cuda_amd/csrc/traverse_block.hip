@@ -474,18 +474,37 @@ __global__ __launch_bounds__(NT, MINW) void traverse_block_kernel(QueryArgs a, B
 #pragma unroll
             for (int u = 0; u < kUnroll; u++) r[u] = *ptr[u];
         };
+        // Per visit four vector instructions and one atomic: a bit-field extract (or a
+        // shift, for the id in the upper half of a word) and a shift-add give the counter
+        // word's LDS address; the id scaled by the field width, taken modulo 32 by the
+        // shift instruction itself, is the field's bit offset.  The sequences are spelled
+        // out because the compiler's canonical form of the same arithmetic is longer.
+        typedef __attribute__((address_space(3))) uint32_t lds_u32;
+        constexpr uint32_t kCs = CBITS == 4 ? 2u : 3u;              // log2(CBITS)
+        const uint32_t field_scale = kCs;                            // SDWA operands cannot be literals
         auto process = [&](const uint4 (&r)[kUnroll], const int (&mr)[kUnroll]) {
 #pragma unroll
             for (int u = 0; u < kUnroll; u++) {
                 if (mr[u] < 0) continue;
-                uint32_t* mcnt = cnt + (size_t)mr[u] * y.wpc;
+                const uint32_t base = (uint32_t)(uintptr_t)(lds_u32*)(cnt + (size_t)mr[u] * y.wpc);
                 const uint32_t w[4] = {r[u].x, r[u].y, r[u].z, r[u].w};
 #pragma unroll
                 for (int e = 0; e < 8; e++) {
-                    const uint32_t local = (w[e >> 1] >> ((e & 1) * 16)) & 0xffffu;
-                    const uint32_t one = 1u << ((local & (kFpw - 1u)) * CBITS);
-                    if (undo) atomicSub(&mcnt[local >> kFshift], one);
-                    else atomicAdd(&mcnt[local >> kFshift], one);
+                    const uint32_t ww = w[e >> 1];
+                    uint32_t word, addr, bit;
+                    if (e & 1) {
+                        word = ww >> (16 + kFshift);
+                        asm("v_lshlrev_b32_sdwa %0, %1, %2 dst_sel:DWORD dst_unused:UNUSED_PAD "
+                            "src0_sel:DWORD src1_sel:WORD_1" : "=v"(bit) : "s"(field_scale), "v"(ww));
+                    } else {
+                        asm("v_bfe_u32 %0, %1, %2, %3" : "=v"(word) : "v"(ww), "n"(kFshift), "n"(16 - kFshift));
+                        bit = ww << kCs;
+                    }
+                    asm("v_lshl_add_u32 %0, %1, 2, %2" : "=v"(addr) : "v"(word), "v"(base));
+                    const uint32_t one = 1u << (bit & 31u);
+                    lds_u32* p = (lds_u32*)(uintptr_t)addr;
+                    if (undo) __hip_atomic_fetch_sub(p, one, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
+                    else __hip_atomic_fetch_add(p, one, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
                 }
             }
         };
