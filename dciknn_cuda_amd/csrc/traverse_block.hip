@@ -508,17 +508,27 @@ __global__ __launch_bounds__(NT, MINW) void traverse_block_kernel(QueryArgs a, B
                 }
             }
         };
-        // two register sets: the reads of one batch are in flight while the other is counted
-        uint4 r_a[kUnroll], r_b[kUnroll];
-        int m_a[kUnroll], m_b[kUnroll];
         constexpr int kBatch = NT * kUnroll;
-        if (total > 0) fetch(0, r_a, m_a);
-        for (int g0 = 0; g0 < total; g0 += 2 * kBatch) {
-            if (g0 + kBatch < total) fetch(g0 + kBatch, r_b, m_b);
-            process(r_a, m_a);
-            if (g0 + kBatch < total) {
-                if (g0 + 2 * kBatch < total) fetch(g0 + 2 * kBatch, r_a, m_a);
-                process(r_b, m_b);
+        if constexpr (MINW <= 4) {
+            // two register sets: the reads of one batch are in flight while the other is counted
+            uint4 r_a[kUnroll], r_b[kUnroll];
+            int m_a[kUnroll], m_b[kUnroll];
+            if (total > 0) fetch(0, r_a, m_a);
+            for (int g0 = 0; g0 < total; g0 += 2 * kBatch) {
+                if (g0 + kBatch < total) fetch(g0 + kBatch, r_b, m_b);
+                process(r_a, m_a);
+                if (g0 + kBatch < total) {
+                    if (g0 + 2 * kBatch < total) fetch(g0 + 2 * kBatch, r_a, m_a);
+                    process(r_b, m_b);
+                }
+            }
+        } else {
+            // tight register budgets: one set; the other workgroups of the CU cover the reads
+            uint4 r_a[kUnroll];
+            int m_a[kUnroll];
+            for (int g0 = 0; g0 < total; g0 += kBatch) {
+                fetch(g0, r_a, m_a);
+                process(r_a, m_a);
             }
         }
         unsigned long long streamed = 0;
