@@ -423,7 +423,12 @@ __global__ __launch_bounds__(NT, MINW) void traverse_block_kernel(QueryArgs a, B
             s_pref[S] = acc_chunks;
         }
         __syncthreads();
-        const uint4* all = reinterpret_cast<const uint4*>(a.lids);
+        // (explicitly global: through a generic pointer the reads would also count as LDS
+        //  traffic and every wait on LDS would wait for them)
+        typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
+        typedef __attribute__((address_space(1))) const u32x4 g_u32x4;
+        typedef __attribute__((address_space(3))) uint32_t lds_u32;
+        g_u32x4* all = (g_u32x4*)a.lids;
         // partial chunks: the first and the last chunk of every range
         if (tid < 2 * S) {
             const int s = tid >> 1;
@@ -431,7 +436,7 @@ __global__ __launch_bounds__(NT, MINW) void traverse_block_kernel(QueryArgs a, B
             const int which = tid & 1;                 // 0 = first chunk, 1 = last chunk
             if (nch > which) {
                 const int cidx = which ? nch - 1 : 0;
-                const uint4 r = all[s_chunk0[s] + cidx];
+                const u32x4 r = all[s_chunk0[s] + cidx];
                 const int pos0 = s_pos0[s] + (cidx << 3);
                 const int ra = s_ra[s], rb = s_rb[s];
                 const int m = (s >> 1) / a.L;
@@ -451,25 +456,26 @@ __global__ __launch_bounds__(NT, MINW) void traverse_block_kernel(QueryArgs a, B
         // a batch are all formed before its reads are issued, and the reads themselves are
         // unconditional (a thread past the end re-reads the first chunk and ignores it), so
         // they go out back to back.
-        int cur = 0, next_pref = s_pref[1], mof = s_mof[0];
+        auto counters_of = [&](int sidx) {      // LDS byte address of the stream's composite's counters
+            return (uint32_t)(uintptr_t)(lds_u32*)(cnt + (size_t)s_mof[sidx] * y.wpc);
+        };
+        int cur = 0, next_pref = s_pref[1];
+        uint32_t cbase = counters_of(0);
         long long delta = s_chunk0[0] + 1 - s_pref[0];      // chunk number -> index into `all`
-        auto fetch = [&](int g0, uint4 (&r)[kUnroll], int (&mr)[kUnroll]) {
-            const uint4* ptr[kUnroll];
+        auto fetch = [&](int g0, u32x4 (&r)[kUnroll], uint32_t (&mr)[kUnroll]) {
+            g_u32x4* ptr[kUnroll];
 #pragma unroll
             for (int u = 0; u < kUnroll; u++) {
                 const int g = g0 + u * NT + tid;
-                mr[u] = -1;
-                ptr[u] = all;
-                if (g < total) {
-                    while (g >= next_pref) {
-                        cur++;
-                        next_pref = s_pref[cur + 1];
-                        mof = s_mof[cur];
-                        delta = s_chunk0[cur] + 1 - s_pref[cur];
-                    }
-                    mr[u] = mof;
-                    ptr[u] = all + (delta + g);
+                const int gg = min(g, total - 1);
+                while (gg >= next_pref) {
+                    cur++;
+                    next_pref = s_pref[cur + 1];
+                    cbase = counters_of(cur);
+                    delta = s_chunk0[cur] + 1 - s_pref[cur];
                 }
+                mr[u] = g < total ? cbase : 0u;          // 0: past the end, nothing to count
+                ptr[u] = all + (delta + gg);
             }
 #pragma unroll
             for (int u = 0; u < kUnroll; u++) r[u] = *ptr[u];
@@ -479,14 +485,13 @@ __global__ __launch_bounds__(NT, MINW) void traverse_block_kernel(QueryArgs a, B
         // word's LDS address; the id scaled by the field width, taken modulo 32 by the
         // shift instruction itself, is the field's bit offset.  The sequences are spelled
         // out because the compiler's canonical form of the same arithmetic is longer.
-        typedef __attribute__((address_space(3))) uint32_t lds_u32;
         constexpr uint32_t kCs = CBITS == 4 ? 2u : 3u;              // log2(CBITS)
         const uint32_t field_scale = kCs;                            // SDWA operands cannot be literals
-        auto process = [&](const uint4 (&r)[kUnroll], const int (&mr)[kUnroll]) {
+        auto process = [&](const u32x4 (&r)[kUnroll], const uint32_t (&mr)[kUnroll]) {
 #pragma unroll
             for (int u = 0; u < kUnroll; u++) {
-                if (mr[u] < 0) continue;
-                const uint32_t base = (uint32_t)(uintptr_t)(lds_u32*)(cnt + (size_t)mr[u] * y.wpc);
+                if (mr[u] == 0u) continue;
+                const uint32_t base = mr[u];
                 const uint32_t w[4] = {r[u].x, r[u].y, r[u].z, r[u].w};
 #pragma unroll
                 for (int e = 0; e < 8; e++) {
@@ -511,8 +516,8 @@ __global__ __launch_bounds__(NT, MINW) void traverse_block_kernel(QueryArgs a, B
         constexpr int kBatch = NT * kUnroll;
         if constexpr (MINW <= 4) {
             // two register sets: the reads of one batch are in flight while the other is counted
-            uint4 r_a[kUnroll], r_b[kUnroll];
-            int m_a[kUnroll], m_b[kUnroll];
+            u32x4 r_a[kUnroll], r_b[kUnroll];
+            uint32_t m_a[kUnroll], m_b[kUnroll];
             if (total > 0) fetch(0, r_a, m_a);
             for (int g0 = 0; g0 < total; g0 += 2 * kBatch) {
                 if (g0 + kBatch < total) fetch(g0 + kBatch, r_b, m_b);
@@ -524,8 +529,8 @@ __global__ __launch_bounds__(NT, MINW) void traverse_block_kernel(QueryArgs a, B
             }
         } else {
             // tight register budgets: one set; the other workgroups of the CU cover the reads
-            uint4 r_a[kUnroll];
-            int m_a[kUnroll];
+            u32x4 r_a[kUnroll];
+            uint32_t m_a[kUnroll];
             for (int g0 = 0; g0 < total; g0 += kBatch) {
                 fetch(g0, r_a, m_a);
                 process(r_a, m_a);
