@@ -656,7 +656,7 @@ __global__ __launch_bounds__(NT, MINW) void traverse_block_kernel(QueryArgs a, B
                 const int lo = s_cprev[sidx], len = s_c[sidx] - lo;
                 if (len >= 32) {
                     probes++;
-                    s_samp[sidx * 16 + t] = stream_prio_bits(load_stream(sidx), lo + (int)(((int64_t)len * t) >> 4));
+                    s_samp[sidx * 16 + t] = stream_prio_bits(load_stream(sidx), lo + (int)(((uint32_t)len * (uint32_t)t) >> 4));
                 }
             }
             __syncthreads();
@@ -730,16 +730,18 @@ __global__ __launch_bounds__(NT, MINW) void traverse_block_kernel(QueryArgs a, B
                         lo[u] = s_cprev[sidx]; hi[u] = s_c[sidx];
                         const int len = hi[u] - lo[u];
                         if (len >= 32) {
+                            // the samples ascend: the number of them ordered before the window
+                            // is the last such sample's index (independent reads, no search)
                             const uint32_t* tab = s_samp + sidx * 16;
-                            int tl = 0, th = 15;
-                            while (tl < th) {
-                                const int mid = (tl + th + 1) >> 1;
-                                const uint32_t v = tab[mid];
-                                if (strict[u] ? v < w_bits : v <= w_bits) tl = mid; else th = mid - 1;
+                            int tl = 0;
+#pragma unroll
+                            for (int t2 = 1; t2 < 16; t2++) {
+                                const uint32_t v = tab[t2];
+                                tl += (strict[u] ? v < w_bits : v <= w_bits) ? 1 : 0;
                             }
                             const int base0 = lo[u];
-                            if (tl > 0) lo[u] = base0 + (int)(((int64_t)len * tl) >> 4) + 1;
-                            if (tl < 15) hi[u] = base0 + (int)(((int64_t)len * (tl + 1)) >> 4);
+                            if (tl > 0) lo[u] = base0 + (int)(((uint32_t)len * (uint32_t)tl) >> 4) + 1;
+                            if (tl < 15) hi[u] = base0 + (int)(((uint32_t)len * (uint32_t)(tl + 1)) >> 4);
                         }
                     }
                     for (;;) {
