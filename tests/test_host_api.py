@@ -135,3 +135,13 @@ def test_workload_generators_are_seeded():
     x4, _ = workloads.c4(n=500, nq=5)
     assert x4.shape == (500, 960)
     assert workloads.c5_batch(0, n=100).shape == (100, 64)
+
+
+def test_bench_refuses_more_than_one_gpu():
+    """bench.py is a one-GPU benchmark: --gpus N > 1 exits with a message, before any GPU work."""
+    import subprocess
+    import sys
+    r = subprocess.run([sys.executable, os.path.join(ROOT, "bench.py"), "--gpus", "2"],
+                       capture_output=True, text=True, timeout=120)
+    assert r.returncode != 0
+    assert "ONE GPU" in r.stderr and r.stdout.strip() == ""
