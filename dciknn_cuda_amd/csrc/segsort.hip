@@ -109,7 +109,8 @@ constexpr int kRadixMax = 63 * 512;
 constexpr int kRadixMin = 512;        // up to this the bitonic tile kernel is faster
 
 template <int kRadixThreads, int IPT>
-__global__ __launch_bounds__(kRadixThreads) void segsort_radix_kernel(
+// (256 threads with more than 45 items each: registers for two workgroups per CU)
+__global__ __launch_bounds__(kRadixThreads, (kRadixThreads == 256 && IPT > 45) ? 2 : 1) void segsort_radix_kernel(
     const float* __restrict__ keys, SegGeom g, float* __restrict__ skeys,
     int32_t* __restrict__ sids, uint32_t* __restrict__ inv, uint16_t* __restrict__ lids) {
     extern __shared__ uint32_t rs[];
@@ -389,7 +390,8 @@ int segsort(const float* d_keys, int num_indices, int64_t n, int block_size,
         DCIH_RADIX(64, 9); DCIH_RADIX(64, 17); DCIH_RADIX(64, 25); DCIH_RADIX(64, 33);
         DCIH_RADIX(128, 21); DCIH_RADIX(128, 27); DCIH_RADIX(128, 33);
         DCIH_RADIX(256, 21); DCIH_RADIX(256, 27); DCIH_RADIX(256, 33); DCIH_RADIX(256, 39); DCIH_RADIX(256, 45);
-        DCIH_RADIX(512, 27); DCIH_RADIX(512, 33); DCIH_RADIX(512, 39); DCIH_RADIX(512, 45);
+        DCIH_RADIX(256, 51); DCIH_RADIX(256, 57);      // two workgroups share a CU: one's passes cover the other's loads and stores
+        DCIH_RADIX(512, 33); DCIH_RADIX(512, 39); DCIH_RADIX(512, 45);
         DCIH_RADIX(512, 51); DCIH_RADIX(512, 57); DCIH_RADIX(512, 63);
 #undef DCIH_RADIX
     }
