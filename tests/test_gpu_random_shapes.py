@@ -2,6 +2,8 @@
 small seeded shapes, including the awkward corners (L = 1, where every visit is a
 promotion; duplicated points, where priorities tie everywhere; windows wider
 than a partition; budgets of 0 and 1 iterations; tiny max_num_candidates)."""
+import os
+
 import numpy as np
 import pytest
 import torch
@@ -44,12 +46,16 @@ def _points(rng, n, nq, dim, kind):
     return x.astype(np.float32), q.astype(np.float32)
 
 
-@pytest.mark.parametrize("seed", range(150))
+# DCIH_RANDOM_SHAPES=<count> widens the sweep for a one-off soak
+@pytest.mark.parametrize("seed", range(int(os.environ.get("DCIH_RANDOM_SHAPES", "150"))))
 def test_random_shape(gpu, oracle, seed):
     from dciknn_cuda_amd import _capi
     rng = np.random.default_rng(1000 + seed)
     M, L, n, B, T, k, outer, max_cand, dim, kind = _shape(rng)
     nq = 6
+    if seed % 10 == 9:      # a larger index and more queries: several epochs, learnt epoch sizes, undos
+        n, nq = int(rng.choice([20000, 50000])), 24
+        k = int(rng.choice([1, 10, 40]))
     X, Q = _points(rng, n, nq, dim, kind)
     xd, qd = torch.from_numpy(X).cuda(), torch.from_numpy(Q).cuda()
     ref = None
