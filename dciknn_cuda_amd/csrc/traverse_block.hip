@@ -191,6 +191,8 @@ __device__ inline int group_partition_point(int lo, int hi, bool active, int lg,
     }
     return lo;
 }
+// x^y for x > 0 from the hardware's log2 / exp2 approximations (epoch sizing only)
+__device__ inline float fast_pow(float x, float y) { return __builtin_amdgcn_exp2f(__builtin_amdgcn_logf(x) * y); }
 __host__ __device__ inline int floor_log2(int v) { int l = 0; while ((2 << l) <= v) l++; return l; }
 
 // MINW = waves per SIMD the register allocation must leave room for: LDS decides how
@@ -314,10 +316,11 @@ __global__ __launch_bounds__(NT, MINW) void traverse_block_kernel(QueryArgs a, B
     const float hint = a.stop_hint ? a.stop_hint[b] : 0.0f;
     const float hint_promos = a.stop_hint ? a.stop_hint[a.B + b] : 0.0f;
     const float kHintFirst = fminf(1.05f,
-        powf(kPromoAim / fmaxf(1.0f, hint_promos > 0.0f ? hint_promos : (float)a.k * (float)T), inv_L));
+        fast_pow(kPromoAim / fmaxf(1.0f, hint_promos > 0.0f ? hint_promos : (float)a.k * (float)T), inv_L));
     {
-        int first = 4;
-        for (int s = 0; s < S; s++) first = max(first, s_ns[s] / 128);
+        int first = 4;           // (every wavefront reduces the S <= 128 stream lengths on its own)
+        for (int s = lane; s < S; s += kWave) first = max(first, s_ns[s] / 128);
+        for (int o = kWave / 2; o > 0; o >>= 1) first = max(first, __shfl_xor(first, o, kWave));
         if (hint > 0.0f) first = max(first, (int)(kHintFirst * hint / (float)(2 * a.L)));
         if (tid < S) s_stride[tid] = first;
         if (tid < a.M) s_Kprev[tid] = 0;
@@ -536,9 +539,10 @@ __global__ __launch_bounds__(NT, MINW) void traverse_block_kernel(QueryArgs a, B
                 process(r_a, m_a);
             }
         }
-        unsigned long long streamed = 0;
-        for (int s = 0; s < S; s++) streamed += (unsigned long long)max(0, s_rb[s] - s_ra[s]);
-        return streamed;
+        long long mine = 0;             // (summed per wavefront: the same total on every thread)
+        for (int s = lane; s < S; s += kWave) mine += (long long)max(0, s_rb[s] - s_ra[s]);
+        for (int o = kWave / 2; o > 0; o >>= 1) mine += __shfl_xor(mine, o, kWave);
+        return (unsigned long long)mine;
     };
 
     unsigned long long streamed = 0;     // entries streamed so far (same on every thread)
@@ -776,13 +780,13 @@ __global__ __launch_bounds__(NT, MINW) void traverse_block_kernel(QueryArgs a, B
         // ---- 5. replay promotions in (step, composite) order ----------------------
         const int ne = (int)misc[kEventCount];
         unsigned long long H = ~0ull;        // steps below H are complete for every composite
-        for (int m = 0; m < a.M; m++) {
-            bool exhausted = true;
-            for (int h = 0; h < 2 * a.L; h++) {
+        for (int m = 0; m < a.M; m++) {      // (the lanes of a wavefront share a composite's streams)
+            bool mine = true;
+            for (int h = lane; h < 2 * a.L; h += kWave) {
                 const int sidx = 2 * m * a.L + h;
-                exhausted = exhausted && s_c[sidx] >= s_ns[sidx];
+                mine = mine && s_c[sidx] >= s_ns[sidx];
             }
-            if (!exhausted) H = min(H, (unsigned long long)s_K[m]);
+            if (!__all(mine)) H = min(H, (unsigned long long)s_K[m]);
         }
         if (ne > 0) {
             int np2 = 2;
@@ -880,9 +884,9 @@ __global__ __launch_bounds__(NT, MINW) void traverse_block_kernel(QueryArgs a, B
         }
         phase(7);
         if (stop) break;
-        bool exhausted_all = true;
-        for (int s = 0; s < S; s++) exhausted_all = exhausted_all && s_c[s] >= s_ns[s];
-        if (exhausted_all) break;     // H was unbounded: everything has been replayed
+        bool mine_exhausted = true;     // every wavefront looks at all S <= 128 streams, a lane at two
+        for (int s = lane; s < S; s += kWave) mine_exhausted = mine_exhausted && s_c[s] >= s_ns[s];
+        if (__all(mine_exhausted)) break;     // H was unbounded: everything has been replayed
         {
             uint32_t kmax = 0, dk_lead = 1;
             for (int m = 0; m < a.M; m++)
@@ -896,7 +900,7 @@ __global__ __launch_bounds__(NT, MINW) void traverse_block_kernel(QueryArgs a, B
                 k_target = fmaxf(t_armed + 1.0f, need) + (float)S;
             } else if (hint > 0.0f) {
                 const float so_far = (float)max(1u, misc[kNumCand] + misc[kEventCount]);   // promotions up to here
-                const float grow = fminf(kHintGrow, powf(1.0f + kPromoAim / so_far, inv_L));
+                const float grow = fminf(kHintGrow, fast_pow(1.0f + kPromoAim / so_far, inv_L));
                 k_target = (float)kmax < 0.9f * kHintFirst * hint ? kHintFirst * hint : grow * (float)kmax + (float)S;
             }
             k_target = fminf(k_target, 2.0f * (float)kmax + 16.0f * (float)S);
