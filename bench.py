@@ -1,4 +1,3 @@
-#!/usr/bin/env python3
 """Benchmark of the Prioritized DCI hot path on one MI355X.
 
     python bench.py [--gpus 1] [--steps K] [--warmup W] [--config c2]
@@ -8,7 +7,12 @@ A step is one pass of the query path (query projection, traversal, exact
 distances, top-k) over the whole seeded query batch of the workload, with the
 index built and all inputs resident in HBM.  The build (projection + segmented
 sort) is timed separately and reported as build_points_per_s.  Prints ONE JSON
-line; see DESIGN.md for the meaning of every field.
+line: value = queries/s; recall_at_k against exact brute force; per_query = exact
+traversal counters of the reference algorithm on a query sample; kernel_ms and
+build = HIP-event times inside the library; roofline = the traversal kernel's
+algorithmic bytes (by the reference's 8-byte index entries) over its time, with
+the measured HBM traffic beside it; cpu_baseline = the CPU restatement of the
+reference algorithm on this box's host cores, on a bounded query sample.
 """
 import argparse
 import json
