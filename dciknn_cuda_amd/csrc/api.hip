@@ -376,6 +376,7 @@ int dcih_query(dcih_index* h, int dim, int num_queries, const float* d_query,
     a.N = h->n;
     a.ppb = (h->n + block_size - 1) / block_size;
     a.dim = dim; a.M = h->M; a.L = h->L; a.B = block_size; a.T = thread_size;
+    a.T_magic = thread_size > 1 ? (unsigned)((0x100000000ull + (unsigned)thread_size - 1u) / (unsigned)thread_size) : 0u;
     a.nq = num_queries; a.k = num_neighbours;
     a.kcap = (int)std::min<int64_t>(num_neighbours, a.ppb);
     a.stop_at = (int64_t)num_outer_iterations * h->L;

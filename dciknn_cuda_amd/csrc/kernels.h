@@ -33,6 +33,7 @@ struct QueryArgs {
     int64_t N;
     int64_t ppb;             // points per partition = ceil(N / B)
     int dim, M, L, B, T, nq, k;
+    unsigned T_magic;        // ceil(2^32 / T) for T > 1: d / T == mulhi(d, T_magic) for 0 <= d < 65536
     int kcap;                // min(k, ppb): results kept per (query, partition)
     int64_t stop_at;         // num_outer_iterations * L
     int64_t max_cand;

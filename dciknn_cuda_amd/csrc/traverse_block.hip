@@ -268,6 +268,10 @@ __global__ __launch_bounds__(NT, MINW) void traverse_block_kernel(QueryArgs a, B
         return;
     }
     const int T = a.T;
+    // d / T for 0 <= d < 65536 (positions inside a partition) by one multiply-high:
+    // exact because the error of the rounded-up reciprocal stays below 2^-16 < 1/T
+    const uint32_t T_magic = a.T_magic;
+    auto div_T = [&](int d) { return T > 1 ? (int)__umulhi((uint32_t)d, T_magic) : d; };
 
     // ---- set-up ---------------------------------------------------------------
     for (int w = tid; w < y.counter_words; w += NT) cnt[w] = 0;
@@ -687,10 +691,10 @@ __global__ __launch_bounds__(NT, MINW) void traverse_block_kernel(QueryArgs a, B
                     int side, j, t, kp;
                     if (pos > p) {
                         const int d = pos - (p + 1);
-                        side = 1; j = d / T; t = d - j * T; kp = p + 1 + j * T;
+                        side = 1; j = div_T(d); t = d - j * T; kp = p + 1 + j * T;
                     } else {
                         const int d = p - pos;
-                        side = 0; j = d / T;
+                        side = 0; j = div_T(d);
                         const int start = p - T + 1 - j * T;
                         t = pos - start; kp = max(start, 0);
                     }
