@@ -782,7 +782,7 @@ __global__ __launch_bounds__(NT, MINW) void traverse_block_kernel(QueryArgs a, B
         if (misc[kFail]) break;
 
         // ---- 5. replay promotions in (step, composite) order ----------------------
-        const int ne = (int)misc[kEventCount];
+        const int ne = __builtin_amdgcn_readfirstlane((int)misc[kEventCount]);
         unsigned long long H = ~0ull;        // steps below H are complete for every composite
         for (int m = 0; m < a.M; m++) {      // (the lanes of a wavefront share a composite's streams)
             bool mine = true;
@@ -798,7 +798,77 @@ __global__ __launch_bounds__(NT, MINW) void traverse_block_kernel(QueryArgs a, B
             for (int j = ne + tid; j < np2; j += NT) events[j] = ~0ull;
             bitonic_sort_u64(events, np2);
         }
-        if (tid == 0) {
+        if (ne <= kWave && wave == 0) {
+            // Up to one event per lane: the walk below is the same as the serial one after
+            // it, but reads steps and flags from registers (lane reads, ballots) instead of
+            // LDS, one dependent round trip per event less; what it accepts is stored by
+            // all lanes together afterwards.
+            const bool have = lane < ne;
+            const unsigned long long ev = have ? events[lane] : ~0ull;
+            const uint32_t ev_t = (uint32_t)(ev >> 32);          // steps fit 32 bits (checked by the host)
+            const uint32_t ev_e = (uint32_t)ev;
+            const uint32_t local = ev_e & 0x1ffffffu;
+            const bool pre = have && ((seen[local >> 5] >> (local & 31u)) & 1u);
+            bool dup = false;      // the same point earlier in the list (promoted under another composite)
+            for (int j = 0; j + 1 < ne; j++) {
+                const uint32_t lj = (uint32_t)__builtin_amdgcn_readlane((int)local, j);
+                dup = dup || (lane > j && lj == local);
+            }
+            const unsigned long long fresh_mask = __ballot(have && !pre && !dup);
+            const unsigned long long lane0_mask = __ballot(have && (ev_e & (1u << 25)));
+            // (first-lane reads tell the compiler that the walk's state is the same on every lane)
+            auto uni = [](uint32_t v) { return (uint32_t)__builtin_amdgcn_readfirstlane((int)v); };
+            long long c0 = (long long)uni(misc[kC0]);
+            bool armed = uni(misc[kArmed]) != 0;
+            unsigned long long t_armed = ((unsigned long long)uni(misc[kArmedHi]) << 32) | uni(misc[kArmedLo]);
+            bool stop = false;
+            unsigned long long kk_star = 0;
+            const unsigned long long last_needed = a.stop_at > 0 ? (unsigned long long)(a.stop_at - 1) : 0ull;
+            int idx = 0;
+            while (idx < ne) {
+                const unsigned long long t = (uint32_t)__builtin_amdgcn_readlane((int)ev_t, idx);
+                if (t >= H) break;
+                if (armed) {
+                    const unsigned long long cand = max(t_armed, last_needed);
+                    if (cand < t) { stop = true; kk_star = cand; break; }
+                }
+                // all events of step t
+                while (idx < ne && (uint32_t)__builtin_amdgcn_readlane((int)ev_t, idx) == (uint32_t)t) {
+                    if ((fresh_mask >> idx) & (lane0_mask >> idx) & 1ull) c0++;
+                    idx++;
+                }
+                if (c0 >= a.k) {
+                    if (!armed) { armed = true; t_armed = t; }
+                    if (c0 >= a.max_cand || (long long)(t + 1) >= a.stop_at) { stop = true; kk_star = t; break; }
+                }
+            }
+            if (!stop && armed) {
+                const unsigned long long cand = max(t_armed, last_needed);
+                if (cand < H) { stop = true; kk_star = cand; }
+            }
+            // events [0, idx) were walked: the fresh ones among them are accepted
+            const unsigned long long walked = idx >= kWave ? ~0ull : ((1ull << idx) - 1ull);
+            const unsigned long long take = fresh_mask & walked;
+            const uint32_t nacc0 = misc[kAccCount], ncand0 = misc[kNumCand];
+            if ((take >> lane) & 1ull) {
+                acc[nacc0 + (uint32_t)__popcll(take & ((1ull << lane) - 1ull))] = local;
+                atomicOr(&seen[local >> 5], 1u << (local & 31u));
+            }
+            // keep what is not settled yet
+            const int keep = stop ? 0 : ne - idx;
+            if (!stop && lane >= idx && have) events[lane - idx] = ev;
+            if (lane == 0) {
+                misc[kEventCount] = (uint32_t)keep;
+                misc[kC0] = (uint32_t)c0;
+                misc[kArmed] = armed ? 1u : 0u;
+                misc[kArmedLo] = (uint32_t)t_armed; misc[kArmedHi] = (uint32_t)(t_armed >> 32);
+                misc[kAccCount] = nacc0 + (uint32_t)__popcll(take);
+                misc[kNumCand] = ncand0 + (uint32_t)__popcll(take);
+                misc[kStop] = stop ? 1u : 0u;
+                misc[kStopStepLo] = (uint32_t)kk_star; misc[kStopStepHi] = (uint32_t)(kk_star >> 32);
+                misc[kPromoCount] = 0;
+            }
+        } else if (ne > kWave && tid == 0) {
             long long c0 = (long long)misc[kC0];
             bool armed = misc[kArmed] != 0;
             unsigned long long t_armed = ((unsigned long long)misc[kArmedHi] << 32) | misc[kArmedLo];
