@@ -671,9 +671,9 @@ __global__ __launch_bounds__(NT, MINW) void traverse_block_kernel(QueryArgs a, B
         }
         {
             // Eight lanes rank one promotion, so 32 promotions are in flight per
-            // workgroup; each lane runs the binary searches of up to four streams in
+            // workgroup; each lane runs the binary searches of up to three streams in
             // lockstep so that their key reads overlap.
-            constexpr int kGroup = 8, kPerLane = 4;
+            constexpr int kGroup = 8, kPerLane = 3;
             const int gl = tid & (kGroup - 1);
             const int group = tid / kGroup;
             for (uint32_t pi = group; pi < np; pi += NT / kGroup) {
