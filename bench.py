@@ -12,7 +12,8 @@ traversal counters of the reference algorithm on a query sample; kernel_ms and
 build = HIP-event times inside the library; roofline = the traversal kernel's
 algorithmic bytes (by the reference's 8-byte index entries) over its time, with
 the measured HBM traffic beside it; cpu_baseline = the CPU restatement of the
-reference algorithm on this box's host cores, on a bounded query sample.
+reference algorithm on this box's host cores, on a bounded query sample; blind =
+the same batch queried blind (candidate ids by promoting step, no distances).
 """
 import argparse
 import json
@@ -239,6 +240,19 @@ def main():
     cm = ctr.double().mean(0).cpu().numpy()
     V, C, S, steps_q = (float(v) for v in cm)
 
+    # ---- blind querying of the same shape (outside the headline's timed region) ----
+    # no distances: per query the first min(10k, outer) promoted candidates by promoting step
+    bids, _ = dci.query(Qd, k, cfg["outer"], blind=True, return_int=True)
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(a.steps):
+        bids, _ = dci.query(Qd, k, cfg["outer"], blind=True, return_int=True)
+    torch.cuda.synchronize()
+    blind_ms = (time.perf_counter() - t0) * 1e3 / a.steps
+    hit = (gt.unsqueeze(2) == bids.long().unsqueeze(1)).any(2).float().mean().item()
+    blind = dict(queries_per_s=nq / (blind_ms * 1e-3), ms_per_step=blind_ms,
+                 slots_per_query=int(bids.shape[1]), true_neighbours_among_slots=hit)
+
     # Algorithmic bytes per query as the roofline contract defines them for this
     # path: query row, 8 bytes (key, id) per search probe and per visited entry,
     # one data row per promoted point, k results.  This engine stores ids apart
@@ -322,6 +336,7 @@ def main():
         "kernel_ms": {"traverse": trav_avg_ms, "merge": float(np.mean(merge_ms)),
                       "query_project": float(np.mean(qproj_ms))},
         "build": build,
+        "blind": blind,
         "roofline": roofline,
         "cpu_baseline": cpu,
     }

@@ -149,8 +149,6 @@ class DCI(object):
         if num_neighbours < 0:
             num_neighbours = self.num_points
         self._ensure_positive_integer(num_neighbours)
-        if blind:
-            raise NotImplementedError("blind querying is not available in this build")
         if self.num_points == 0:
             raise RuntimeError("query on an empty DCI instance; call add() first")
         if num_neighbours > self.num_points:
@@ -164,13 +162,16 @@ class DCI(object):
                                             max_num_candidates, self._block_size, self._thread_size)
             half = _query_result.shape[0] // 2
             return _query_result[:half].reshape(nq, -1), _query_result[half:].reshape(nq, -1)
-        ids = torch.empty((nq, num_neighbours), dtype=torch.int32, device=self._device)
-        dists = torch.empty((nq, num_neighbours), dtype=torch.float32, device=self._device)
+        # blind: candidate ids in the order they were promoted and the steps that promoted
+        # them, as many as the reference's result buffer holds (src/dci_cuda_kernel.cu:782-783)
+        width = min(max_num_candidates, num_outer_iterations) if blind else num_neighbours
+        ids = torch.empty((nq, width), dtype=torch.int32, device=self._device)
+        dists = torch.empty((nq, width), dtype=torch.float32, device=self._device)
         counters = None
         if return_counters:
             counters = torch.empty((nq, _capi.NUM_COUNTERS), dtype=torch.int64, device=self._device)
         _capi.check(self._lib.dcih_query(
-            self._dci_inst, self._dim, nq, _query.data_ptr(), num_neighbours, 0,
+            self._dci_inst, self._dim, nq, _query.data_ptr(), num_neighbours, 1 if blind else 0,
             num_outer_iterations, max_num_candidates, self._block_size, self._thread_size,
             ids.data_ptr(), dists.data_ptr(),
             counters.data_ptr() if counters is not None else None,
@@ -231,8 +232,6 @@ class MDCI(object):
         _query = _query.detach().clone().to(self.dcis[0]._device)
         d0 = self.dcis[0]
         d0._check_data(_query)
-        if blind:
-            raise NotImplementedError("blind querying is not available in this build")
         max_num_candidates = 10 * num_neighbours
         res = _ext._dci_multi_query([dc._capsule for dc in self.dcis], d0._dim, _query.shape[0],
                                     [_query.flatten()], num_neighbours, blind, num_outer_iterations,
@@ -240,6 +239,8 @@ class MDCI(object):
         half = res[0].shape[0] // 2
         nns = res[0][:half].reshape(_query.shape[0], -1)
         dists = res[0][half:].reshape(_query.shape[0], -1)
+        if blind:     # already ordered by promoting step; nothing to merge with one device
+            return nns, dists
         _, sort_indices = torch.sort(dists, dim=1, stable=True)
         sort_indices = sort_indices[:, :num_neighbours]
         return torch.gather(nns, 1, sort_indices), torch.gather(dists, 1, sort_indices)

@@ -11,6 +11,7 @@
 #include <c10/hip/HIPStream.h>
 #include <torch/extension.h>
 
+#include <algorithm>
 #include <stdexcept>
 #include <string>
 #include <vector>
@@ -86,14 +87,19 @@ void dci_add(py::handle capsule, int dim, int64_t num_points, torch::Tensor data
 }
 
 // src/dci_cuda.cpp:84-118 (py_dci_query): flat float32 tensor, first half the ids
-// (as floats, like the reference), second half the distances.
+// (as floats, like the reference), second half the distances.  Blind: per query
+// min(max_num_candidates, num_outer_iterations) candidate ids (the size
+// src/dci_cuda_kernel.cu:775-783 asks for; the reference's own buffer at :99 is
+// too small for it), second half the steps at which they were promoted.
 torch::Tensor dci_query(py::handle capsule, int dim, int num_queries, torch::Tensor query,
                         int num_neighbours, bool blind, int num_outer_iterations,
                         int max_num_candidates, int block_size, int thread_size) {
     require_f32_device(query, "query");
     TORCH_CHECK(query.numel() == (int64_t)num_queries * dim, "query has the wrong number of elements");
     c10::DeviceGuard guard(query.device());
-    const int64_t cells = (int64_t)num_queries * num_neighbours;
+    const int64_t per_query = blind ? std::min(max_num_candidates, num_outer_iterations) : num_neighbours;
+    TORCH_CHECK(per_query > 0, "nothing to return per query");
+    const int64_t cells = (int64_t)num_queries * per_query;
     auto ids = torch::empty({cells}, query.options().dtype(torch::kInt32));
     auto dists = torch::empty({cells}, query.options());
     check(dcih_query(index_of(capsule), dim, num_queries, query.data_ptr<float>(), num_neighbours,

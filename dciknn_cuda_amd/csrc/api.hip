@@ -346,13 +346,17 @@ int dcih_query(dcih_index* h, int dim, int num_queries, const float* d_query,
                int max_num_candidates, int block_size, int thread_size,
                int32_t* d_nn, float* d_dists, uint64_t* d_counters, void* stream) {
     if (!h) return fail(DCIH_EINVAL, "dcih_query: null handle");
-    if (blind) return fail(DCIH_EUNSUPPORTED, "dcih_query: blind querying is not built");
     if (dim != h->dim) return fail(DCIH_EINVAL, "dcih_query: dim differs from the index's");
     if (h->n <= 0) return fail(DCIH_ESTATE, "dcih_query: index is empty");
     if (num_neighbours <= 0 || num_neighbours > h->n)
         return fail(DCIH_EINVAL, "dcih_query: num_neighbours must be in [1, num_points]");
-    if (num_queries < 0 || (num_queries > 0 && (!d_query || !d_nn || !d_dists)))
+    if (num_queries < 0 || (num_queries > 0 && (!d_query || !d_nn || (!blind && !d_dists))))
         return fail(DCIH_EINVAL, "dcih_query: null buffer");
+    // blind: as many candidates per query as the reference's result buffer holds (:782-783)
+    const int64_t num_results =
+        blind ? std::min<int64_t>(max_num_candidates, num_outer_iterations) : num_neighbours;
+    if (num_results <= 0)
+        return fail(DCIH_EINVAL, "dcih_query: blind querying needs positive max_num_candidates and num_outer_iterations");
     if (thread_size <= 0) return fail(DCIH_EINVAL, "dcih_query: thread_size must be positive");
     if (block_size != h->block_size)
         return fail(DCIH_EINVAL, "dcih_query: block_size differs from the one the index was built with");
@@ -377,8 +381,9 @@ int dcih_query(dcih_index* h, int dim, int num_queries, const float* d_query,
     a.ppb = (h->n + block_size - 1) / block_size;
     a.dim = dim; a.M = h->M; a.L = h->L; a.B = block_size; a.T = thread_size;
     a.T_magic = thread_size > 1 ? (unsigned)((0x100000000ull + (unsigned)thread_size - 1u) / (unsigned)thread_size) : 0u;
-    a.nq = num_queries; a.k = num_neighbours;
-    a.kcap = (int)std::min<int64_t>(num_neighbours, a.ppb);
+    a.nq = num_queries; a.k = (int)std::min<int64_t>(num_results, 0x7fffffff);
+    a.k_stop = num_neighbours; a.blind = blind ? 1 : 0;
+    a.kcap = (int)std::min<int64_t>(num_results, a.ppb);
     a.stop_at = (int64_t)num_outer_iterations * h->L;
     a.max_cand = max_num_candidates;
     a.counters = (unsigned long long*)d_counters;

@@ -32,12 +32,15 @@ struct QueryArgs {
     const float* qproj;      // [I][nq]
     int64_t N;
     int64_t ppb;             // points per partition = ceil(N / B)
-    int dim, M, L, B, T, nq, k;
+    int dim, M, L, B, T, nq;
+    int k;                   // results per query
+    int k_stop;              // promotions by a window's first lane that arm the stop rule (num_neighbours)
+    int blind;               // 1: a candidate is scored by the step that promoted it, no distance is computed
     unsigned T_magic;        // ceil(2^32 / T) for T > 1: d / T == mulhi(d, T_magic) for 0 <= d < 65536
     int kcap;                // min(k, ppb): results kept per (query, partition)
     int64_t stop_at;         // num_outer_iterations * L
     int64_t max_cand;
-    unsigned long long* part;      // [nq][B][kcap] packed (dist bits << 32 | id)
+    unsigned long long* part;      // [nq][B][kcap] packed (dist bits << 32 | id); blind: (step << 32 | id)
     unsigned long long* counters;  // null or [nq][4]
     uint32_t* gscratch;      // global visit counters when they do not fit LDS
     int32_t* redo_items;     // [nq*B] (query, partition) pairs the batch kernel hands back
@@ -48,7 +51,7 @@ struct QueryArgs {
     unsigned long long* phase_ticks;  // null, or 16 accumulators for the batch kernel's phases
     int mode;                // 0 = pick, 1 = step-by-step kernel, 2 = batch kernel
     int32_t* out_ids;        // [nq][k]
-    float* out_dists;        // [nq][k]
+    float* out_dists;        // [nq][k]; blind: null, or the promoting steps as floats
 };
 size_t query_part_bytes(const QueryArgs& a);
 // Bytes of global counter scratch the traversal needs (0 when LDS suffices).

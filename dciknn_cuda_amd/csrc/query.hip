@@ -200,13 +200,17 @@ __global__ __launch_bounds__(kWave) void traverse_kernel(QueryArgs a, Layout y) 
                         const int src = __ffsll((long long)pm) - 1;
                         pm &= pm - 1;
                         const int cpt = __shfl(pt, src, kWave);
-                        // exact distance (:36-44), row read by the whole wavefront
-                        const float* const rows1[1] = {a.data + (int64_t)cpt * a.dim};
-                        float dist1[1];
-                        wave_row_dists<1>(rows1, s_q, a.dim, rows_vec4(a.data, a.dim), dist1);
-                        const float dist = dist1[0];
-                        const unsigned long long e =
-                            ((unsigned long long)__builtin_bit_cast(uint32_t, dist) << 32) | (uint32_t)cpt;
+                        uint32_t score;
+                        if (a.blind) {
+                            score = (uint32_t)kk;     // (:498-505: recorded, no distance)
+                        } else {
+                            // exact distance (:36-44), row read by the whole wavefront
+                            const float* const rows1[1] = {a.data + (int64_t)cpt * a.dim};
+                            float dist1[1];
+                            wave_row_dists<1>(rows1, s_q, a.dim, rows_vec4(a.data, a.dim), dist1);
+                            score = __builtin_bit_cast(uint32_t, dist1[0]);
+                        }
+                        const unsigned long long e = ((unsigned long long)score << 32) | (uint32_t)cpt;
                         ncand++;
                         if (t0 + src == 0) c0++;          // only lane 0's promotions count (:413, :598)
                         if (tk_count < a.kcap) {
@@ -243,7 +247,7 @@ __global__ __launch_bounds__(kWave) void traverse_kernel(QueryArgs a, Layout y) 
                 __syncthreads();
             }
             steps++;
-            if (c0 >= a.k && (kk + 1 >= a.stop_at || c0 >= a.max_cand)) break;   // :598-607
+            if (c0 >= a.k_stop && (kk + 1 >= a.stop_at || c0 >= a.max_cand)) break;   // :598-607
             if (!any) break;   // every simple index exhausted: nothing can change any more
             kk++;
         }
@@ -289,8 +293,10 @@ __global__ __launch_bounds__(kMergeThreads) void merge_topk_kernel(QueryArgs a, 
         const unsigned long long v = buf[j];
         const bool empty = v == ~0ull;
         a.out_ids[(int64_t)qi * a.k + j] = empty ? -1 : (int32_t)(uint32_t)v;
-        a.out_dists[(int64_t)qi * a.k + j] =
-            empty ? __builtin_inff() : __builtin_bit_cast(float, (uint32_t)(v >> 32));
+        if (a.out_dists)
+            a.out_dists[(int64_t)qi * a.k + j] =
+                empty ? __builtin_inff()
+                      : (a.blind ? (float)(uint32_t)(v >> 32) : __builtin_bit_cast(float, (uint32_t)(v >> 32)));
     }
 }
 
@@ -327,7 +333,11 @@ size_t query_gscratch_bytes(const QueryArgs& a) {
 int query(const QueryArgs& a_in, hipStream_t s, hipEvent_t* ev) {
     QueryArgs a = a_in;
     if (a.nq <= 0) return 0;
-    if (a.k > 8192) return fail(-4, "query: num_neighbours above 8192 is not supported");
+    if (a.k > 8192)
+        return fail(-4, a.blind ? "query: more than 8192 blind candidates per query are not supported"
+                                : "query: num_neighbours above 8192 is not supported");
+    if (a.blind && (int64_t)a.L * (a.ppb + 2 * (int64_t)a.T) >= 0x7fffffffLL)
+        return fail(-4, "query: blind querying needs step numbers that fit 31 bits");
     if ((int64_t)a.M * a.ppb * 8 > 0x7fffffffLL)
         return fail(-4, "query: partition too large for the visit counters; use a larger block_size");
     const Layout y = make_layout(a);

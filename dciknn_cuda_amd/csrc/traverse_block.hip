@@ -90,7 +90,7 @@ BlockLayout make_block_layout(const QueryArgs& a) {
     // The tables grow with the promotions a stop needs (about k * T, more when the
     // step limit rather than c0 >= k ends the traversal): fewer, larger epochs.
     y.promo_cap = 256;
-    while (y.promo_cap < 2 * (int64_t)a.k * a.T && y.promo_cap < 2048) y.promo_cap <<= 1;
+    while (y.promo_cap < 2 * (int64_t)a.k_stop * a.T && y.promo_cap < 2048) y.promo_cap <<= 1;
     y.promo_max = y.promo_cap * 5 / 8;
     y.event_cap = 2 * y.promo_cap;
     y.sort_cap = 64;           // top-k plus a batch of at least 48 new candidates
@@ -99,7 +99,8 @@ BlockLayout make_block_layout(const QueryArgs& a) {
     // promotion list, both of which the ranking before it has finished with
     y.off_samp = o;
     y.off_acc = o;
-    o += max(2 * I * 16 * 4 + y.promo_cap * 4, y.event_cap * 4);
+    // (blind querying keeps the promoting step beside every accepted candidate)
+    o += max(2 * I * 16 * 4 + y.promo_cap * 4, y.event_cap * 4 * (a.blind ? 2 : 1));
     y.off_promo = y.off_samp + 2 * I * 16 * 4;
     o = (o + 15) & ~15;
     y.off_events = o;   o += y.event_cap * 8;
@@ -226,6 +227,7 @@ __global__ __launch_bounds__(NT, MINW) void traverse_block_kernel(QueryArgs a, B
     uint32_t* s_samp = reinterpret_cast<uint32_t*>(smem + y.off_samp);
     uint32_t* promo = reinterpret_cast<uint32_t*>(smem + y.off_promo);
     uint32_t* acc = reinterpret_cast<uint32_t*>(smem + y.off_acc);
+    uint32_t* acc_step = acc + y.event_cap;       // blind querying only
     unsigned long long* events = reinterpret_cast<unsigned long long*>(smem + y.off_events);
     unsigned long long* sortbuf = reinterpret_cast<unsigned long long*>(smem + y.off_sort);
     uint32_t* cnt = reinterpret_cast<uint32_t*>(smem + y.off_cnt);
@@ -320,7 +322,7 @@ __global__ __launch_bounds__(NT, MINW) void traverse_block_kernel(QueryArgs a, B
     const float hint = a.stop_hint ? a.stop_hint[b] : 0.0f;
     const float hint_promos = a.stop_hint ? a.stop_hint[a.B + b] : 0.0f;
     const float kHintFirst = fminf(1.05f,
-        fast_pow(kPromoAim / fmaxf(1.0f, hint_promos > 0.0f ? hint_promos : (float)a.k * (float)T), inv_L));
+        fast_pow(kPromoAim / fmaxf(1.0f, hint_promos > 0.0f ? hint_promos : (float)a.k_stop * (float)T), inv_L));
     {
         int first = 4;           // (every wavefront reduces the S <= 128 stream lengths on its own)
         for (int s = lane; s < S; s += kWave) first = max(first, s_ns[s] / 128);
@@ -837,7 +839,7 @@ __global__ __launch_bounds__(NT, MINW) void traverse_block_kernel(QueryArgs a, B
                     if ((fresh_mask >> idx) & (lane0_mask >> idx) & 1ull) c0++;
                     idx++;
                 }
-                if (c0 >= a.k) {
+                if (c0 >= a.k_stop) {
                     if (!armed) { armed = true; t_armed = t; }
                     if (c0 >= a.max_cand || (long long)(t + 1) >= a.stop_at) { stop = true; kk_star = t; break; }
                 }
@@ -851,7 +853,9 @@ __global__ __launch_bounds__(NT, MINW) void traverse_block_kernel(QueryArgs a, B
             const unsigned long long take = fresh_mask & walked;
             const uint32_t nacc0 = misc[kAccCount], ncand0 = misc[kNumCand];
             if ((take >> lane) & 1ull) {
-                acc[nacc0 + (uint32_t)__popcll(take & ((1ull << lane) - 1ull))] = local;
+                const uint32_t slot = nacc0 + (uint32_t)__popcll(take & ((1ull << lane) - 1ull));
+                acc[slot] = local;
+                if (a.blind) acc_step[slot] = ev_t;
                 atomicOr(&seen[local >> 5], 1u << (local & 31u));
             }
             // keep what is not settled yet
@@ -892,13 +896,14 @@ __global__ __launch_bounds__(NT, MINW) void traverse_block_kernel(QueryArgs a, B
                     const uint32_t bit = 1u << (local & 31);
                     if (!(seen[local >> 5] & bit)) {
                         seen[local >> 5] |= bit;
+                        if (a.blind) acc_step[nacc] = (uint32_t)t;
                         acc[nacc++] = local;
                         ncand++;
                         if (e & (1u << 25)) c0++;
                     }
                     idx++;
                 }
-                if (c0 >= a.k) {
+                if (c0 >= a.k_stop) {
                     if (!armed) { armed = true; t_armed = t; }
                     if (c0 >= a.max_cand || (long long)(t + 1) >= a.stop_at) { stop = true; kk_star = t; break; }
                 }
@@ -929,9 +934,13 @@ __global__ __launch_bounds__(NT, MINW) void traverse_block_kernel(QueryArgs a, B
         for (int done = 0; done < nacc;) {      // in batches that fit beside the top-k
             const int topn = (int)misc[kTopN];
             const int batch = min(nacc - done, y.sort_cap - topn);
+            if (a.blind) {      // scored by the promoting step (:498-505), no row is read
+                for (int c = tid; c < batch; c += NT)
+                    sortbuf[topn + c] = ((unsigned long long)acc_step[done + c] << 32) | (uint32_t)(off + acc[done + c]);
+            }
             // two candidates per wavefront at a time: their row reads overlap
             const bool vec4 = rows_vec4(a.data, a.dim);
-            for (int c = wave; c < batch; c += 2 * kWaves) {
+            for (int c = wave; c < (a.blind ? 0 : batch); c += 2 * kWaves) {
                 const int c2 = c + kWaves;
                 const int64_t pt0 = off + acc[done + c];
                 const int64_t pt1 = c2 < batch ? off + acc[done + c2] : pt0;

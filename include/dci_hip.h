@@ -115,14 +115,26 @@ int dcih_append(dcih_index* h, int dim, int64_t num_points, const float* d_data,
                 int block_size, int thread_size, void* stream);
 
 /*
- * Replaces dci_query (include/dci.h:71, src/dci_cuda_kernel.cu:777-875) with
- * query_config.blind == false.  d_query is [num_queries][dim]; for each query
+ * Replaces dci_query (include/dci.h:71, src/dci_cuda_kernel.cu:777-875).
+ * d_query is [num_queries][dim]; with blind == 0, for each query
  * d_nn / d_dists [num_queries][num_neighbours] receive the ids and Euclidean
  * distances of the num_neighbours best promoted candidates, ascending by
  * (distance, id); slots beyond the number of candidates get id -1 and +inf.
  * block_size must equal the value given to dcih_add (the partitioning is part
  * of the built index); thread_size is the window width.  d_counters is NULL or
- * [num_queries][DCIH_NUM_COUNTERS].  blind != 0 returns DCIH_EUNSUPPORTED.
+ * [num_queries][DCIH_NUM_COUNTERS].
+ *
+ * blind != 0 (query_config.blind, :498-505, :754-773, :859-864): the same
+ * traversal under the same stop rule, but no distance is computed.  d_nn is
+ * [num_queries][R] with R = min(max_num_candidates, num_outer_iterations), the
+ * size the reference asks of its caller (:775-776, :782-783), and receives the
+ * ids of the first R promoted candidates of the query, ascending by (outer step
+ * of its partition's traversal at which the point was promoted, id), then -1.
+ * d_dists may be NULL (:776); if not, it is [num_queries][R] and receives those
+ * step numbers as floats (+inf beside -1).  The reference ranks blind
+ * candidates by a count that is 1 for every one of them and collects them
+ * through per-thread cursors that overwrite each other, so it defines no order;
+ * this one does.  R above 8192 returns DCIH_EUNSUPPORTED.
  */
 int dcih_query(dcih_index* h, int dim, int num_queries, const float* d_query,
                int num_neighbours, int blind, int num_outer_iterations,

@@ -110,9 +110,12 @@ inline float window_priority(const float* key, int n, int T, int* cur, float q) 
     return kInf;
 }
 
-struct Cand { float dist; int id; };
-inline bool cand_less(const Cand& a, const Cand& b) {
-    return a.dist < b.dist || (a.dist == b.dist && a.id < b.id);
+/* A candidate and what ranks it: its distance, or, in blind querying, the
+ * outer step of its partition's traversal that promoted it. */
+template <class Score> struct Cand { Score score; int id; };
+template <class Score>
+inline bool cand_less(const Cand<Score>& a, const Cand<Score>& b) {
+    return a.score < b.score || (a.score == b.score && a.id < b.id);
 }
 
 struct Scratch {
@@ -125,10 +128,12 @@ struct Scratch {
 struct Stats { uint64_t visited = 0, cands = 0, probes = 0, steps = 0; };
 
 /* One partition of one query: src/dci_cuda_kernel.cu:401-626 with
- * blockIdx.x = b, blockDim.x = T.  Emits (dist, id) for every promoted point. */
+ * blockIdx.x = b, blockDim.x = T.  Emits (id, outer step) for every promoted
+ * point; the caller computes the distance (:506-511) or, blind, records the
+ * point (:498-505). */
 template <class Emit>
-void traverse_partition(const float* skeys, const int* sids, const float* data,
-                        const float* q, const float* qp, int64_t N, int dim,
+void traverse_partition(const float* skeys, const int* sids,
+                        const float* qp, int64_t N,
                         int M, int L, int T, int64_t seg_off, int n, int k,
                         int64_t outer, int64_t max_cand, Scratch& s, Stats& st,
                         Emit emit) {
@@ -178,7 +183,7 @@ void traverse_partition(const float* skeys, const int* sids, const float* data,
                 if (++cnt[local] == L && !s.seen[local]) {
                     s.seen[local] = 1;
                     st.cands++;
-                    emit(euclid(data + (int64_t)pt * dim, q, dim), pt);
+                    emit(pt, kk);
                     if (t == 0) c0++;
                 }
             }
@@ -275,6 +280,84 @@ int dci_oracle_window_sequence(const float* key, int n, int T, float q,
     return cnt;
 }
 
+}  // extern "C"
+
+namespace {
+
+/* Shared body of the two query entry points below.  BLIND == false: the k_out
+ * best of all promoted candidates by (distance, id), src/dci_cuda_kernel.cu
+ * :506-554 and :691-701.  BLIND == true: the first k_out of them by (promoting
+ * step, id), see dci_oracle_query_blind. */
+template <bool BLIND, class Score>
+int query_impl(const float* skeys, const int* sids, const float* data,
+               const float* query, const float* qproj, int64_t N, int dim,
+               int M, int L, int B, int T, int nq, int k, int64_t k_out,
+               int64_t outer, int64_t max_cand, int* out_ids, Score* out_scores,
+               Score empty_score, uint64_t* counters, int* cand_ids,
+               int64_t cand_cap, int64_t* cand_cnt, int num_threads) {
+    if (k <= 0 || k > N || k_out <= 0 || B <= 0 || T <= 0 || M <= 0 || L <= 0 || L > 65535) return -1;
+    const int I = M * L;
+    const int64_t ppb = (N + B - 1) / B;   /* :424 */
+#ifdef _OPENMP
+    if (num_threads > 0) omp_set_num_threads(num_threads);
+#endif
+#pragma omp parallel
+    {
+        Scratch s;
+        std::vector<Cand<Score>> heap;  /* max-heap of the k_out best so far */
+#pragma omp for schedule(dynamic, 1)
+        for (int j = 0; j < nq; j++) {
+            heap.clear();
+            Stats st;
+            int64_t ncand = 0;
+            const float* q = query + (int64_t)j * dim;
+            const float* qp = qproj + (int64_t)j * I;
+            for (int b = 0; b < B; b++) {
+                const int64_t off = (int64_t)b * ppb;
+                const int64_t n = std::min(N - off, ppb);   /* :425-427 */
+                if (n <= 0) continue;                       /* :429 */
+                traverse_partition(
+                    skeys, sids, qp, N, M, L, T, off, (int)n, k,
+                    outer, max_cand, s, st, [&](int id, int64_t step) {
+                        if (cand_ids && ncand < cand_cap)
+                            cand_ids[(int64_t)j * cand_cap + ncand] = id;
+                        ncand++;
+                        Cand<Score> c;
+                        if constexpr (BLIND) c.score = (Score)step;
+                        else c.score = euclid(data + (int64_t)id * dim, q, dim);
+                        c.id = id;
+                        if ((int64_t)heap.size() < k_out) {
+                            heap.push_back(c);
+                            std::push_heap(heap.begin(), heap.end(), cand_less<Score>);
+                        } else if (cand_less(c, heap.front())) {
+                            std::pop_heap(heap.begin(), heap.end(), cand_less<Score>);
+                            heap.back() = c;
+                            std::push_heap(heap.begin(), heap.end(), cand_less<Score>);
+                        }
+                    });
+            }
+            std::sort_heap(heap.begin(), heap.end(), cand_less<Score>);
+            for (int64_t r = 0; r < k_out; r++) {
+                const bool have = r < (int64_t)heap.size();
+                out_ids[(int64_t)j * k_out + r] = have ? heap[r].id : -1;
+                if (out_scores) out_scores[(int64_t)j * k_out + r] = have ? heap[r].score : empty_score;
+            }
+            if (counters) {
+                counters[(int64_t)j * 4 + 0] = st.visited;
+                counters[(int64_t)j * 4 + 1] = st.cands;
+                counters[(int64_t)j * 4 + 2] = st.probes;
+                counters[(int64_t)j * 4 + 3] = st.steps;
+            }
+            if (cand_cnt) cand_cnt[j] = ncand;
+        }
+    }
+    return 0;
+}
+
+}  // namespace
+
+extern "C" {
+
 /* src/dci_cuda_kernel.cu:777-865 (dci_query) over src/dci_cuda_kernel.cu:401-626
  * per (query, partition), then the k best of the union (:691-701).
  *
@@ -295,64 +378,37 @@ int dci_oracle_query(const float* skeys, const int* sids, const float* data,
                      int64_t max_cand, int* out_ids, float* out_dists,
                      uint64_t* counters, int* cand_ids, int64_t cand_cap,
                      int64_t* cand_cnt, int num_threads) {
-    if (k <= 0 || k > N || B <= 0 || T <= 0 || M <= 0 || L <= 0 || L > 65535) return -1;
-    const int I = M * L;
-    const int64_t ppb = (N + B - 1) / B;   /* :424 */
-#ifdef _OPENMP
-    if (num_threads > 0) omp_set_num_threads(num_threads);
-#endif
-#pragma omp parallel
-    {
-        Scratch s;
-        std::vector<Cand> heap;  /* max-heap of the k best so far */
-#pragma omp for schedule(dynamic, 1)
-        for (int j = 0; j < nq; j++) {
-            heap.clear();
-            Stats st;
-            int64_t ncand = 0;
-            const float* q = query + (int64_t)j * dim;
-            const float* qp = qproj + (int64_t)j * I;
-            for (int b = 0; b < B; b++) {
-                const int64_t off = (int64_t)b * ppb;
-                const int64_t n = std::min(N - off, ppb);   /* :425-427 */
-                if (n <= 0) continue;                       /* :429 */
-                traverse_partition(
-                    skeys, sids, data, q, qp, N, dim, M, L, T, off, (int)n, k,
-                    outer, max_cand, s, st, [&](float dist, int id) {
-                        if (cand_ids && ncand < cand_cap)
-                            cand_ids[(int64_t)j * cand_cap + ncand] = id;
-                        ncand++;
-                        Cand c{dist, id};
-                        if ((int)heap.size() < k) {
-                            heap.push_back(c);
-                            std::push_heap(heap.begin(), heap.end(), cand_less);
-                        } else if (cand_less(c, heap.front())) {
-                            std::pop_heap(heap.begin(), heap.end(), cand_less);
-                            heap.back() = c;
-                            std::push_heap(heap.begin(), heap.end(), cand_less);
-                        }
-                    });
-            }
-            std::sort_heap(heap.begin(), heap.end(), cand_less);
-            for (int r = 0; r < k; r++) {
-                if (r < (int)heap.size()) {
-                    out_ids[(int64_t)j * k + r] = heap[r].id;
-                    out_dists[(int64_t)j * k + r] = heap[r].dist;
-                } else {
-                    out_ids[(int64_t)j * k + r] = -1;
-                    out_dists[(int64_t)j * k + r] = kInf;
-                }
-            }
-            if (counters) {
-                counters[(int64_t)j * 4 + 0] = st.visited;
-                counters[(int64_t)j * 4 + 1] = st.cands;
-                counters[(int64_t)j * 4 + 2] = st.probes;
-                counters[(int64_t)j * 4 + 3] = st.steps;
-            }
-            if (cand_cnt) cand_cnt[j] = ncand;
-        }
-    }
-    return 0;
+    return query_impl<false, float>(skeys, sids, data, query, qproj, N, dim, M, L, B, T, nq, k, k,
+                                    outer, max_cand, out_ids, out_dists, kInf, counters,
+                                    cand_ids, cand_cap, cand_cnt, num_threads);
+}
+
+/*
+ * Blind querying: dci_query with query_config.blind == true
+ * (src/dci_cuda_kernel.cu:498-505 records a promoted point instead of computing
+ * its distance; :754-773 and :859-864 return max_possible_num_candidates =
+ * min(max_num_candidates, num_outer_iterations) ids per query, :782-783).  The
+ * traversal and its stop rule (:598-607, armed by k = num_neighbours) are those
+ * of dci_oracle_query.  The reference ranks the recorded points by how often
+ * they were recorded, which is once each (a point belongs to one partition and
+ * :497 admits it once), and records them through per-thread cursors that
+ * overwrite each other (:500-504), so it fixes no order among them.  This
+ * restatement fixes one: ascending by (outer step kk of the partition's
+ * traversal at which the point was promoted, id).
+ *
+ *   out_ids   : [nq][R], R = min(max_cand, outer); -1 beyond the candidates
+ *   out_steps : nullable [nq][R]; 0xffffffff beside -1
+ * Returns 0, or -1 on invalid arguments.
+ */
+int dci_oracle_query_blind(const float* skeys, const int* sids,
+                           const float* qproj, int64_t N,
+                           int M, int L, int B, int T, int nq, int k, int64_t outer,
+                           int64_t max_cand, int* out_ids, uint32_t* out_steps,
+                           uint64_t* counters, int num_threads) {
+    const int64_t R = std::min(max_cand, outer);
+    return query_impl<true, uint32_t>(skeys, sids, nullptr, nullptr, qproj, N, 0, M, L, B, T, nq,
+                                      k, R, outer, max_cand, out_ids, out_steps, 0xffffffffu,
+                                      counters, nullptr, 0, nullptr, num_threads);
 }
 
 int dci_oracle_max_threads(void) {

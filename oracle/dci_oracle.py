@@ -54,6 +54,11 @@ def lib():
             ctypes.c_void_p, ctypes.c_void_p, ctypes.c_int64, ctypes.c_void_p,
             ctypes.c_int]
         L.dci_oracle_query.restype = ctypes.c_int
+        L.dci_oracle_query_blind.argtypes = [
+            _f32p, _i32p, _f32p, ctypes.c_int64, ctypes.c_int, ctypes.c_int,
+            ctypes.c_int, ctypes.c_int, ctypes.c_int, ctypes.c_int, ctypes.c_int64,
+            ctypes.c_int64, _i32p, ctypes.c_void_p, ctypes.c_void_p, ctypes.c_int]
+        L.dci_oracle_query_blind.restype = ctypes.c_int
         L.dci_oracle_max_threads.argtypes = []
         L.dci_oracle_max_threads.restype = ctypes.c_int
         _lib = L
@@ -135,6 +140,33 @@ def query(skeys, sids, data, queries, qproj, M, L, B, T, k, outer,
         raise ValueError("dci_oracle_query rejected its arguments")
     return dict(ids=ids, dists=dists, counters=counters, cand_ids=cand_ids,
                 cand_cnt=cand_cnt)
+
+
+def query_blind(skeys, sids, qproj, M, L, B, T, k, outer, max_cand=None,
+                num_threads=0):
+    """Blind query: dict(ids, steps, counters), [nq][min(max_cand, outer)] each.
+
+    ids are the promoted points ascending by (promoting step, id), -1 beyond
+    them; steps the promoting steps (uint32, all ones beside -1).
+    """
+    skeys, qproj = _f32(skeys), _f32(qproj)
+    sids = np.ascontiguousarray(sids, dtype=np.int32)
+    N = skeys.shape[1]
+    nq = qproj.shape[0]
+    assert skeys.shape == (M * L, N) and sids.shape == (M * L, N)
+    assert qproj.shape == (nq, M * L)
+    if max_cand is None:
+        max_cand = 10 * k
+    R = min(max_cand, outer)
+    ids = np.empty((nq, R), np.int32)
+    steps = np.empty((nq, R), np.uint32)
+    counters = np.zeros((nq, 4), np.uint64)
+    rc = lib().dci_oracle_query_blind(
+        skeys, sids, qproj, N, M, L, B, T, nq, k, outer, max_cand, ids,
+        steps.ctypes.data, counters.ctypes.data, num_threads)
+    if rc != 0:
+        raise ValueError("dci_oracle_query_blind rejected its arguments")
+    return dict(ids=ids, steps=steps, counters=counters)
 
 
 def build_index(P, X, block_size):

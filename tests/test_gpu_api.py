@@ -103,8 +103,6 @@ def test_argument_errors(gpu):
         dci.query(Q, 0)
     with pytest.raises(ValueError):
         dci.query(Q, 2001)
-    with pytest.raises(NotImplementedError):
-        dci.query(Q, 3, blind=True)
     dci._block_size = 11                                # partitioning is part of the index
     with pytest.raises(RuntimeError):
         dci.query(Q, 3)

@@ -52,6 +52,22 @@ def test_traversal_hand_traces(oracle, case):
     assert r["counters"][:, 3].tolist() == case["steps"]
 
 
+@pytest.mark.parametrize("case", GOLD["blind_traversals"], ids=lambda c: c["name"][:40])
+def test_blind_traversal_hand_traces(oracle, case):
+    P = np.array(case["directions"], f32)
+    X = np.array(case["data"], f32)
+    Q = np.array(case["query"], f32)
+    sk, si = oracle.build_index(P, X, case["B"])
+    r = oracle.query_blind(sk, si, oracle.project(Q, P), case["M"], case["L"], case["B"],
+                           case["T"], case["k"], case["outer"], max_cand=case["max_cand"])
+    assert r["ids"].tolist() == case["ids"]
+    assert r["steps"].astype(np.int64).tolist() == [[s if s >= 0 else 0xffffffff for s in row]
+                                                    for row in case["steps"]]
+    assert r["counters"][:, 0].tolist() == case["visited"]
+    assert r["counters"][:, 1].tolist() == case["candidates"]
+    assert r["counters"][:, 3].tolist() == case["num_steps"]
+
+
 # ------------------------------------------------------------ library routines
 def test_search_is_searchsorted_left_minus_one(oracle):
     rng = np.random.default_rng(0)
@@ -213,7 +229,7 @@ def _index_windows(key, T, q):
     return out
 
 
-def _rank_model(sk, si, qp, n_off, n, M, L, T, k, outer, max_cand):
+def _rank_model(sk, si, qp, n_off, n, M, L, T, k, outer, max_cand, with_times=False):
     """Promotion events of one partition without running the step loop.
     Composite m consumes its windows in ascending (priority, simple index,
     own order); a point's promotion time under m is the largest rank among the
@@ -269,6 +285,8 @@ def _rank_model(sk, si, qp, n_off, n, M, L, T, k, outer, max_cand):
     end = stop if stop is not None else last_step
     cands = [pt for (t, m, pt, l0) in events if t <= end]
     visited = sum(sum(v[:end + 1]) for v in visited_at)
+    if with_times:
+        return [(t, pt) for (t, m, pt, l0) in events if t <= end]
     return cands, visited, end + 1
 
 
@@ -312,6 +330,72 @@ def test_rank_model_agrees_with_oracle(oracle, case):
         d = np.sqrt(((X[cands].astype(np.float64) - Q[j].astype(np.float64)) ** 2).sum(1))
         best = [cands[t] for t in np.argsort(d, kind="stable")[:k]]
         assert set(r["ids"][j].tolist()) - {-1} == set(best)
+
+
+@pytest.mark.parametrize("case", MODEL_CASES, ids=[str(c) for c in MODEL_CASES])
+@pytest.mark.parametrize("max_cand", [None, 3])
+def test_rank_model_agrees_with_blind_oracle(oracle, case, max_cand):
+    """Blind result = the model's promotion events of all partitions sorted by
+    (time, id), cut to min(max_cand, outer) slots."""
+    seed, n, dim, M, L, B, T, k, outer = case
+    if max_cand is None:
+        max_cand = 10 * k
+    rng = np.random.default_rng(seed)
+    X = rng.standard_normal((n, dim)).astype(f32)
+    Q = rng.standard_normal((5, dim)).astype(f32)
+    P = oracle.normalize(rng.standard_normal((M * L, dim)).astype(f32))
+    sk, si = oracle.build_index(P, X, B)
+    qp = oracle.project(Q, P)
+    r = oracle.query_blind(sk, si, qp, M, L, B, T, k, outer, max_cand=max_cand)
+    R = min(max_cand, outer)
+    assert r["ids"].shape == (5, R)
+    ppb = -(-n // B)
+    for j in range(5):
+        ev = []
+        for b in range(B):
+            off = b * ppb
+            nb = min(n - off, ppb)
+            if nb > 0:
+                ev += _rank_model(sk, si, qp[j], off, nb, M, L, T, k, outer, max_cand, with_times=True)
+        ev.sort()
+        assert int(r["counters"][j, 1]) == len(ev)
+        want_ids = [pt for _, pt in ev][:R] + [-1] * max(0, R - len(ev))
+        want_steps = [t for t, _ in ev][:R] + [0xffffffff] * max(0, R - len(ev))
+        assert r["ids"][j].tolist() == want_ids
+        assert r["steps"][j].astype(np.int64).tolist() == want_steps
+
+
+def test_blind_candidates_are_the_query_candidates(oracle):
+    """The blind ids are points whose distances the ordinary query computes (all of
+    them when they fit the slots), in step order, and the counters coincide."""
+    rng = np.random.default_rng(21)
+    n, dim, M, L = 1500, 10, 2, 3
+    X = rng.standard_normal((n, dim)).astype(f32)
+    Q = rng.standard_normal((6, dim)).astype(f32)
+    P = oracle.normalize(rng.standard_normal((M * L, dim)).astype(f32))
+    fitted = 0
+    for B, T, k, outer, max_cand in [(1, 1, 6, 100000, 60), (4, 5, 6, 40, 100000), (3, 2, 4, 2000, 25)]:
+        sk, si = oracle.build_index(P, X, B)
+        qp = oracle.project(Q, P)
+        full = oracle.query(sk, si, X, Q, qp, M, L, B, T, k, outer, max_cand=max_cand, cand_cap=n)
+        blind = oracle.query_blind(sk, si, qp, M, L, B, T, k, outer, max_cand=max_cand)
+        np.testing.assert_array_equal(full["counters"], blind["counters"])
+        R = min(max_cand, outer)
+        for j in range(6):
+            nc = int(full["cand_cnt"][j])
+            cands = set(full["cand_ids"][j, :nc].tolist())
+            got = blind["ids"][j]
+            m = min(nc, R)
+            assert set(got[:m].tolist()) <= cands and len(set(got[:m].tolist())) == m
+            assert np.all(got[m:] == -1)
+            if nc <= R:
+                fitted += 1
+                assert set(got[:m].tolist()) == cands
+            st = blind["steps"][j, :m].astype(np.int64)
+            assert np.all(np.diff(st) >= 0)
+            same = np.diff(st) == 0
+            assert np.all(np.diff(got[:m])[same] > 0), "equal steps rank by id"
+    assert fitted > 0
 
 
 # ------------------------------------------------------------------ invariants
