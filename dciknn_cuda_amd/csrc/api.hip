@@ -389,6 +389,30 @@ int dcih_query(dcih_index* h, int dim, int num_queries, const float* d_query,
     a.counters = (unsigned long long*)d_counters;
     a.out_ids = d_nn; a.out_dists = d_dists;
 
+    if (!blind && num_neighbours > 8192) {
+        // Beyond the top-k tables.  With more neighbours asked for than a partition holds, no
+        // partition can stop early (c0 counts promotions of one partition, :598-607), so the
+        // answer is the full ranking and is computed as such.  (With exactly as many, the
+        // results are the same but the last step may end the loop before its idle pass.)
+        if (num_neighbours < a.ppb || (num_neighbours == a.ppb && d_counters))
+            return fail(DCIH_EUNSUPPORTED,
+                        "dcih_query: num_neighbours above 8192 is supported when it exceeds the points "
+                        "per partition (ceil(num_points / block_size)); build with a larger block_size");
+        const int chunk = exhaustive_chunk(h->n, num_queries);
+        const size_t qp_bytes = d_counters ? align_up((size_t)I * num_queries * sizeof(float)) : 0;
+        int rc = ensure_ws(h, qp_bytes + exhaustive_ws_bytes(h->n, chunk));
+        if (rc) return rc;
+        if (d_counters) {
+            rc = project(h->d_dirs, I, d_query, num_queries, dim, (float*)h->ws, s);
+            if (rc) return rc;
+            a.qproj = (float*)h->ws;
+        }
+        mark(h, DCIH_T_TRAVERSE, 0, s);
+        rc = query_exhaustive(a, (char*)h->ws + qp_bytes, chunk, s);
+        mark(h, DCIH_T_TRAVERSE, 1, s);
+        return rc;
+    }
+
     const size_t qp_bytes = align_up((size_t)I * num_queries * sizeof(float));
     const size_t part_bytes = align_up(query_part_bytes(a));
     const size_t gs_bytes = align_up(query_gscratch_bytes(a));

@@ -61,6 +61,14 @@ size_t query_gscratch_bytes(const QueryArgs& a);
 bool block_traversal_supported(const QueryArgs& a, size_t* lds_bytes);
 int query_block(const QueryArgs& a, hipStream_t s);
 
+// Full ranking (exhaustive.hip) for num_neighbours above the points per partition,
+// where the traversal provably visits everything: queries are processed `chunk` at
+// a time in `ws` (exhaustive_ws_bytes(N, chunk) bytes); a.qproj is needed only when
+// a.counters is set.
+int exhaustive_chunk(int64_t N, int nq);
+size_t exhaustive_ws_bytes(int64_t N, int chunk);
+int query_exhaustive(const QueryArgs& a, void* ws, int chunk, hipStream_t s);
+
 // ev: null, or three events recorded before the traversal, between traversal
 // and merge, and after the merge.
 int query(const QueryArgs& a, hipStream_t s, hipEvent_t* ev);

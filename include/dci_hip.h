@@ -124,6 +124,17 @@ int dcih_append(dcih_index* h, int dim, int64_t num_points, const float* d_data,
  * of the built index); thread_size is the window width.  d_counters is NULL or
  * [num_queries][DCIH_NUM_COUNTERS].
  *
+ * num_neighbours may be as large as the number of indexed points (what
+ * dciknn_cuda/core.py:84-85 passes when the caller gives none).  Up to 8192 the
+ * traversal keeps its best candidates in on-chip tables.  Above 8192 it must also
+ * exceed the points per partition, ceil(num_points / block_size): the stop rule
+ * (:598-607) counts promotions of one partition, so it can then never fire, every
+ * point is promoted, and the result, the num_neighbours closest of all points by
+ * (distance, id), is computed directly (all distances, one sort per query; the
+ * counters from their closed forms).  Distances on this path are summed in index
+ * order like compute_dist_device (:36-44).  8192 < num_neighbours <= points per
+ * partition returns DCIH_EUNSUPPORTED (equality is accepted without d_counters).
+ *
  * blind != 0 (query_config.blind, :498-505, :754-773, :859-864): the same
  * traversal under the same stop rule, but no distance is computed.  d_nn is
  * [num_queries][R] with R = min(max_num_candidates, num_outer_iterations), the

@@ -189,3 +189,70 @@ def test_append_equals_one_add_of_the_concatenation(gpu, oracle):
     fresh.add(X)
     d = fresh.query(Q, 8, 40, return_int=True)
     assert torch.equal(d[0], want[0])
+
+
+# ------------------------------------------------ num_neighbours beyond the top-k tables
+def _full_ranking_case(gpu, oracle, n, nq, dim, M, L, B, T, k, outer=50, seed=8):
+    rng = np.random.default_rng(seed)
+    X = rng.standard_normal((n, dim)).astype(np.float32)
+    Q = rng.standard_normal((nq, dim)).astype(np.float32)
+    dci = gpu.DCI(dim, M, L, B, T, seed=seed)
+    dci.add(torch.from_numpy(X).cuda())
+    ids, dists, ctr = dci.query(torch.from_numpy(Q).cuda(), k, outer, return_int=True, return_counters=True)
+    torch.cuda.synchronize()
+    from util import engine_index, engine_project
+    skeys, sids = engine_index(dci)
+    qproj = engine_project(dci.directions.numpy(), Q).T.copy()
+    kk = n if k < 0 else k
+    ref = oracle.query(skeys, sids, X, Q, qproj, M, L, B, T, kk, outer)
+    dci.free()
+    return ids.cpu().numpy(), dists.cpu().numpy(), ctr.cpu().numpy(), ref, X, Q
+
+
+@pytest.mark.parametrize("n,B,T,k", [(20000, 4, 3, -1), (20000, 4, 1, 9000), (9000, 2, 5, -1),
+                                     (70000, 16, 8, -1), (40000, 5, 2, 8193)])
+def test_full_ranking_beyond_8192(gpu, oracle, n, B, T, k):
+    """num_neighbours above the points per partition (core.py:84-85 makes it num_points by
+    default): no partition can stop early, so the traversal's answer is the exact ranking
+    of all points, which the engine computes directly.  Distances are summed in the
+    oracle's order, so ids, distances and all four counters are compared exactly."""
+    ids, dists, ctr, ref, X, Q = _full_ranking_case(gpu, oracle, n, 3, 12, 2, 3, B, T, k)
+    np.testing.assert_array_equal(ids, ref["ids"])
+    np.testing.assert_array_equal(dists, ref["dists"])
+    np.testing.assert_array_equal(ctr, ref["counters"].astype(np.int64))
+    kk = n if k < 0 else k
+    bi, bd = oracle.brute_force(X, Q, kk)
+    assert set_agreement_rows(ids, bi) >= 0.999
+    np.testing.assert_allclose(dists, bd, rtol=1e-5)
+
+
+def set_agreement_rows(a, b):
+    return float(np.mean([len(set(x.tolist()) & set(y.tolist())) / len(y) for x, y in zip(a, b)]))
+
+
+@pytest.mark.parametrize("B", [10, 1])
+def test_full_ranking_through_the_binding(gpu, B):
+    """The reference's route (flat float tensor from _dci_query) with the default
+    num_neighbours: every point, ranked."""
+    rng = np.random.default_rng(12)
+    X = torch.from_numpy(rng.standard_normal((10000, 8)).astype(np.float32)).cuda()
+    Q = torch.from_numpy(rng.standard_normal((2, 8)).astype(np.float32)).cuda()
+    dci = gpu.DCI(8, 2, 3, B, 4, seed=2)
+    dci.add(X)
+    ids, dists = dci.query(Q)
+    assert ids.shape == (2, 10000) and dists.shape == (2, 10000)
+    assert torch.equal(torch.sort(ids.long(), dim=1).values, torch.arange(10000, device="cuda").expand(2, -1))
+    assert torch.all(dists[:, 1:] >= dists[:, :-1])
+    want = (X[ids.long()] - Q[:, None, :]).norm(dim=2)        # the distance of the id beside it
+    assert torch.allclose(dists, want, rtol=1e-5, atol=1e-6)
+    dci.free()
+
+
+def test_large_k_below_partition_size_is_refused(gpu):
+    rng = np.random.default_rng(13)
+    X = torch.from_numpy(rng.standard_normal((20000, 8)).astype(np.float32)).cuda()
+    dci = gpu.DCI(8, 2, 3, 2, 4, seed=2)      # 10000 points per partition
+    dci.add(X)
+    with pytest.raises(RuntimeError):
+        dci.query(X[:1], 9000)
+    dci.free()

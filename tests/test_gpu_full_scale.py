@@ -82,3 +82,21 @@ def test_more_iterations_never_worse(c2):
         if prev is not None:
             assert torch.all(d <= prev * (1 + 1e-6))
         prev = d
+
+
+def test_full_ranking_of_a_million_points(c2):
+    """num_neighbours left at its default (every point, core.py:84-85) at full size:
+    a permutation of all ids, ascending, each distance that of the id beside it, and
+    the head of the ranking equal to the exact nearest neighbours."""
+    dci, Xd, Qd = c2["dci"], c2["Xd"], c2["Qd"][:3].contiguous()
+    n = Xd.shape[0]
+    ids, dists = dci.query(Qd, -1, OUTER, return_int=True)
+    assert ids.shape == (3, n)
+    assert torch.equal(torch.sort(ids.long(), dim=1).values, torch.arange(n, device="cuda").expand(3, -1))
+    assert torch.all(dists[:, 1:] >= dists[:, :-1])
+    for j in range(3):
+        d = (Xd[ids[j].long()] - Qd[j]).norm(dim=1)
+        assert torch.allclose(d, dists[j], rtol=1e-5, atol=1e-4)
+        exact = (Xd - Qd[j]).norm(dim=1)
+        order = torch.argsort(exact, stable=True)[:100]
+        assert len(set(order.tolist()) & set(ids[j, :100].tolist())) >= 99
