@@ -32,7 +32,7 @@ HBM_PEAK_GBS = 8000.0   # MI355X HBM3E
 # (2.000 and 1.000); the counter runs are summarised in profiles/bench_c2_hbm_traffic.txt.
 # Counters cannot be read from inside this process, so the figure is a constant
 # tied to that exact configuration and omitted for any other.
-MEASURED_TRAFFIC_C2_DEFAULT = 72.6e9
+MEASURED_TRAFFIC_C2_DEFAULT = 62.3e9
 
 # (block_size, thread_size, num_outer_iterations) used when none are given:
 # the fastest setting found with recall@k >= 0.95 on that workload.
@@ -56,7 +56,7 @@ def parse():
     p.add_argument("--outer", type=int)
     p.add_argument("--nq", type=int, help="use only the first NQ queries")
     p.add_argument("--n", type=int, help="override the number of data points")
-    p.add_argument("--cpu-queries", type=int, default=512,
+    p.add_argument("--cpu-queries", type=int, default=2048,
                    help="queries in the CPU baseline sample")
     p.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     p.add_argument("--build-reps", type=int, default=3)
