@@ -367,7 +367,7 @@ int dcih_query(dcih_index* h, int dim, int num_queries, const float* d_query,
 
     QueryArgs a;
     a.skeys = h->d_skeys; a.sids = h->d_sids; a.inv = h->d_inv; a.lids = h->d_lids; a.data = h->d_data; a.query = d_query;
-    a.mode = h->traversal; a.item_list = nullptr; a.item_count = nullptr;
+    a.mode = h->traversal; a.item_list = nullptr; a.item_count = nullptr; a.dense = nullptr;
     a.phase_ticks = h->d_phase_ticks;
     // the hints describe where traversals of one query shape stop; forget them when it changes
     if (h->hint_k != num_neighbours || h->hint_outer != num_outer_iterations ||
@@ -389,15 +389,31 @@ int dcih_query(dcih_index* h, int dim, int num_queries, const float* d_query,
     a.counters = (unsigned long long*)d_counters;
     a.out_ids = d_nn; a.out_dists = d_dists;
 
+    if (num_results > 8192 &&
+        (blind || num_neighbours < a.ppb || (num_neighbours == a.ppb && d_counters))) {
+        // More results than the top-k tables hold while partitions may still stop early: the
+        // step-by-step traversal records every candidate in a dense row per query, which is
+        // then sorted like the full ranking below.
+        const int chunk = exhaustive_chunk(h->n, num_queries);
+        QueryArgs probe = a;
+        probe.nq = chunk; probe.kcap = 1;
+        const size_t qp_bytes = align_up((size_t)I * chunk * sizeof(float));
+        const size_t rank_bytes = align_up(exhaustive_ws_bytes(h->n, chunk));
+        const size_t gs_bytes = align_up(query_gscratch_bytes(probe));
+        int rc = ensure_ws(h, qp_bytes + rank_bytes + gs_bytes);
+        if (rc) return rc;
+        a.gscratch = gs_bytes ? (uint32_t*)((char*)h->ws + qp_bytes + rank_bytes) : nullptr;
+        mark(h, DCIH_T_TRAVERSE, 0, s);
+        rc = query_dense(a, h->d_dirs, h->ws, chunk, s);
+        mark(h, DCIH_T_TRAVERSE, 1, s);
+        return rc;
+    }
     if (!blind && num_neighbours > 8192) {
-        // Beyond the top-k tables.  With more neighbours asked for than a partition holds, no
-        // partition can stop early (c0 counts promotions of one partition, :598-607), so the
-        // answer is the full ranking and is computed as such.  (With exactly as many, the
-        // results are the same but the last step may end the loop before its idle pass.)
-        if (num_neighbours < a.ppb || (num_neighbours == a.ppb && d_counters))
-            return fail(DCIH_EUNSUPPORTED,
-                        "dcih_query: num_neighbours above 8192 is supported when it exceeds the points "
-                        "per partition (ceil(num_points / block_size)); build with a larger block_size");
+        // With more neighbours asked for than a partition holds, no partition can stop early
+        // (c0 counts promotions of one partition, :598-607), so the answer is the full ranking
+        // and is computed as such.  (With exactly as many, the results are the same but the
+        // last step may end the loop before its idle pass: the counters then come from the
+        // traversal above.)
         const int chunk = exhaustive_chunk(h->n, num_queries);
         const size_t qp_bytes = d_counters ? align_up((size_t)I * num_queries * sizeof(float)) : 0;
         int rc = ensure_ws(h, qp_bytes + exhaustive_ws_bytes(h->n, chunk));

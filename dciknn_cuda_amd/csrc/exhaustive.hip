@@ -59,15 +59,24 @@ __global__ __launch_bounds__(kExThreads) void exact_dists_kernel(
         if (q0 + j < nq) out[(int64_t)(q0 + j) * N + row] = (float)sqrt((double)acc[j]);
 }
 
-// The first k columns of every sorted row.
+// The first k columns of every sorted row.  Columns past the end of a row and, when
+// asked, entries whose value is +inf (points that never became candidates) read as
+// "no result": id -1, +inf.
 __global__ __launch_bounds__(256) void take_columns_kernel(
     const float* __restrict__ skeys, const int32_t* __restrict__ sids, int64_t N, int k,
-    int32_t* __restrict__ out_ids, float* __restrict__ out_dists) {
+    int inf_is_empty, int32_t* __restrict__ out_ids, float* __restrict__ out_vals) {
     const int q = blockIdx.y;
     for (int j = blockIdx.x * 256 + threadIdx.x; j < k; j += gridDim.x * 256) {
-        out_ids[(int64_t)q * k + j] = sids[(int64_t)q * N + j];
-        out_dists[(int64_t)q * k + j] = skeys[(int64_t)q * N + j];
+        const float v = j < N ? skeys[(int64_t)q * N + j] : __builtin_inff();
+        const bool empty = j >= N || (inf_is_empty && v == __builtin_inff());
+        out_ids[(int64_t)q * k + j] = empty ? -1 : sids[(int64_t)q * N + j];
+        if (out_vals) out_vals[(int64_t)q * k + j] = v;
     }
+}
+
+__global__ void fill_f32_kernel(float* p, int64_t n, float v) {
+    const int64_t stride = (int64_t)gridDim.x * blockDim.x;
+    for (int64_t e = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; e < n; e += stride) p[e] = v;
 }
 
 // Counters of a traversal that runs every partition dry, one wavefront per
@@ -134,16 +143,36 @@ size_t exhaustive_ws_bytes(int64_t N, int chunk) {
     return 3 * align256(cells * 4) + align256(segsort_tmp_bytes(chunk, N, 1));
 }
 
+float* rank_rows_input(void* ws) { return (float*)ws; }
+
+int fill_rows(float* d_rows, int64_t cells, float value, hipStream_t s) {
+    hipLaunchKernelGGL(fill_f32_kernel, dim3((unsigned)min((int64_t)8192, (cells + 255) / 256)), dim3(256), 0, s,
+                       d_rows, cells, value);
+    DCIH_HIP(hipGetLastError());
+    return 0;
+}
+
+int rank_rows(void* ws, int chunk, int rows, int64_t N, int k, bool inf_is_empty,
+              int32_t* out_ids, float* out_vals, hipStream_t s) {
+    const size_t cells = (size_t)chunk * (size_t)N;
+    char* base = (char*)ws;
+    float* d_in = (float*)base;
+    float* d_sorted = (float*)(base + align256(cells * 4));
+    int32_t* d_sids = (int32_t*)(base + 2 * align256(cells * 4));
+    void* d_tmp = segsort_tmp_bytes(chunk, N, 1) ? (void*)(base + 3 * align256(cells * 4)) : nullptr;
+    const int rc = segsort(d_in, rows, N, 1, d_sorted, d_sids, nullptr, nullptr, d_tmp, s);
+    if (rc) return rc;
+    hipLaunchKernelGGL(take_columns_kernel, dim3((unsigned)min(1024, (k + 255) / 256), (unsigned)rows),
+                       dim3(256), 0, s, d_sorted, d_sids, N, k, inf_is_empty ? 1 : 0, out_ids, out_vals);
+    DCIH_HIP(hipGetLastError());
+    return 0;
+}
+
 int query_exhaustive(const QueryArgs& a, void* ws, int chunk, hipStream_t s) {
     if (a.nq <= 0) return 0;
     if ((a.N + kExThreads - 1) / kExThreads > 0x7fffffffLL || (int64_t)a.nq * a.B > 0x7fffffffLL)
         return fail(-4, "query: too many points for the full-ranking path");
-    const size_t cells = (size_t)chunk * (size_t)a.N;
-    char* base = (char*)ws;
-    float* d_dist = (float*)base;
-    float* d_sdist = (float*)(base + align256(cells * 4));
-    int32_t* d_sids = (int32_t*)(base + 2 * align256(cells * 4));
-    void* d_tmp = segsort_tmp_bytes(chunk, a.N, 1) ? (void*)(base + 3 * align256(cells * 4)) : nullptr;
+    float* d_dist = rank_rows_input(ws);
     for (int q0 = 0; q0 < a.nq; q0 += chunk) {
         const int nqc = min(chunk, a.nq - q0);
         hipLaunchKernelGGL(exact_dists_kernel,
@@ -152,12 +181,9 @@ int query_exhaustive(const QueryArgs& a, void* ws, int chunk, hipStream_t s) {
                            dim3(kExThreads), 0, s, a.data, a.N, a.dim,
                            a.query + (int64_t)q0 * a.dim, nqc, d_dist);
         DCIH_HIP(hipGetLastError());
-        const int rc = segsort(d_dist, nqc, a.N, 1, d_sdist, d_sids, nullptr, nullptr, d_tmp, s);
+        const int rc = rank_rows(ws, chunk, nqc, a.N, a.k, false, a.out_ids + (int64_t)q0 * a.k,
+                                 a.out_dists + (int64_t)q0 * a.k, s);
         if (rc) return rc;
-        hipLaunchKernelGGL(take_columns_kernel, dim3((unsigned)min(1024, (a.k + 255) / 256), (unsigned)nqc),
-                           dim3(256), 0, s, d_sdist, d_sids, a.N, a.k,
-                           a.out_ids + (int64_t)q0 * a.k, a.out_dists + (int64_t)q0 * a.k);
-        DCIH_HIP(hipGetLastError());
     }
     if (a.counters) {
         const int64_t cellsc = (int64_t)a.nq * 4;

@@ -52,6 +52,7 @@ struct QueryArgs {
     int mode;                // 0 = pick, 1 = step-by-step kernel, 2 = batch kernel
     int32_t* out_ids;        // [nq][k]
     float* out_dists;        // [nq][k]; blind: null, or the promoting steps as floats
+    float* dense;            // null, or [nq][N]: the step-by-step kernel stores every candidate's score here instead of keeping a top-k
 };
 size_t query_part_bytes(const QueryArgs& a);
 // Bytes of global counter scratch the traversal needs (0 when LDS suffices).
@@ -68,6 +69,18 @@ int query_block(const QueryArgs& a, hipStream_t s);
 int exhaustive_chunk(int64_t N, int nq);
 size_t exhaustive_ws_bytes(int64_t N, int chunk);
 int query_exhaustive(const QueryArgs& a, void* ws, int chunk, hipStream_t s);
+// The pieces of it that the dense-row traversal (query_dense) shares: rows of N values
+// at rank_rows_input(ws), `rows` <= chunk of them; rank_rows sorts every row by (value,
+// column) and writes the first k columns (id = column, or -1 for +inf when asked).
+float* rank_rows_input(void* ws);
+int fill_rows(float* d_rows, int64_t cells, float value, hipStream_t s);
+int rank_rows(void* ws, int chunk, int rows, int64_t N, int k, bool inf_is_empty,
+              int32_t* out_ids, float* out_vals, hipStream_t s);
+// More results per query than the top-k tables hold, early stops possible: the
+// step-by-step kernel writes every candidate's score into a dense row of its query
+// (+inf = not a candidate), rank_rows does the rest.  Projects the queries itself
+// (d_dirs), chunk by chunk; ws = I*chunk floats + exhaustive_ws_bytes(N, chunk) bytes.
+int query_dense(const QueryArgs& a, const float* d_dirs, void* ws, int chunk, hipStream_t s);
 
 // ev: null, or three events recorded before the traversal, between traversal
 // and merge, and after the merge.

@@ -120,7 +120,8 @@ __global__ __launch_bounds__(kWave) void traverse_kernel(QueryArgs a, Layout y) 
         unsigned long long* top = y.topk_bytes ? s_top : a.part + item * a.kcap;
         unsigned long long* part_out = a.part + item * a.kcap;
         if (n <= 0) {   // empty partition (src/dci_cuda_kernel.cu:429)
-            for (int j = lane; j < a.kcap; j += kWave) part_out[j] = ~0ull;
+            if (!a.dense)
+                for (int j = lane; j < a.kcap; j += kWave) part_out[j] = ~0ull;
             continue;
         }
         uint32_t* cnt = LDS_COUNTERS ? s_cnt
@@ -213,7 +214,12 @@ __global__ __launch_bounds__(kWave) void traverse_kernel(QueryArgs a, Layout y) 
                         const unsigned long long e = ((unsigned long long)score << 32) | (uint32_t)cpt;
                         ncand++;
                         if (t0 + src == 0) c0++;          // only lane 0's promotions count (:413, :598)
-                        if (tk_count < a.kcap) {
+                        if (a.dense) {
+                            // every candidate is kept: its score goes to its own cell of the query's row
+                            if (lane == 0)
+                                a.dense[(int64_t)qi * a.N + cpt] =
+                                    a.blind ? (float)score : __builtin_bit_cast(float, score);
+                        } else if (tk_count < a.kcap) {
                             if (lane == 0) top[tk_count] = e;
                             if (tk_count == 0 || e > tk_max) { tk_max = e; tk_maxslot = tk_count; }
                             tk_count++;
@@ -254,7 +260,7 @@ __global__ __launch_bounds__(kWave) void traverse_kernel(QueryArgs a, Layout y) 
 
         __syncthreads();
         if (!y.topk_bytes) __threadfence();
-        for (int j = lane; j < a.kcap; j += kWave) {
+        for (int j = lane; j < (a.dense ? 0 : a.kcap); j += kWave) {
             const unsigned long long v = j < tk_count ? top[j] : ~0ull;
             part_out[j] = v;
         }
@@ -389,6 +395,61 @@ int query(const QueryArgs& a_in, hipStream_t s, hipEvent_t* ev) {
                        (size_t)cap * sizeof(unsigned long long), s, a, cap);
     if (ev) (void)hipEventRecord(ev[2], s);
     DCIH_HIP(hipGetLastError());
+    return 0;
+}
+
+int query_dense(const QueryArgs& a_in, const float* d_dirs, void* ws, int chunk, hipStream_t s) {
+    if (a_in.nq <= 0) return 0;
+    const int I = a_in.M * a_in.L;
+    if ((int64_t)a_in.M * a_in.ppb * 8 > 0x7fffffffLL)
+        return fail(-4, "query: partition too large for the visit counters; use a larger block_size");
+    // blind scores are step numbers stored as floats: they must stay exact
+    if (a_in.blind && (int64_t)a_in.L * (a_in.ppb + 2 * (int64_t)a_in.T) >= (1 << 24))
+        return fail(-4, "query: this many blind results need step numbers below 2^24; use a larger block_size");
+    static bool attr_done = false;
+    if (!attr_done) {
+        DCIH_HIP(hipFuncSetAttribute((const void*)traverse_kernel<true>,
+                                     hipFuncAttributeMaxDynamicSharedMemorySize, kMaxLds));
+        DCIH_HIP(hipFuncSetAttribute((const void*)traverse_kernel<false>,
+                                     hipFuncAttributeMaxDynamicSharedMemorySize, kMaxLds));
+        attr_done = true;
+    }
+    const size_t qp_bytes = ((size_t)I * chunk * sizeof(float) + 255) & ~(size_t)255;
+    float* d_qproj = (float*)ws;
+    void* ws_rank = (char*)ws + qp_bytes;
+    for (int q0 = 0; q0 < a_in.nq; q0 += chunk) {
+        QueryArgs a = a_in;             // this chunk's queries as a query batch of their own
+        a.nq = min(chunk, a_in.nq - q0);
+        a.query = a_in.query + (int64_t)q0 * a.dim;
+        a.qproj = d_qproj;
+        a.counters = a_in.counters ? a_in.counters + (int64_t)q0 * 4 : nullptr;
+        a.kcap = 1;                     // no per-partition lists
+        a.part = nullptr;
+        a.item_list = nullptr;
+        a.item_count = nullptr;
+        a.dense = rank_rows_input(ws_rank);
+        int rc = project(d_dirs, I, a.query, a.nq, a.dim, d_qproj, s);
+        if (rc) return rc;
+        rc = fill_rows(a.dense, (int64_t)a.nq * a.N, __builtin_inff(), s);
+        if (rc) return rc;
+        const Layout y = make_layout(a);
+        if (y.lds_bytes > (size_t)kMaxLds)
+            return fail(-4, "query: dim / num_indices too large for LDS state");
+        const int64_t cells = a.counters ? (int64_t)a.nq * 4 : 0;
+        hipLaunchKernelGGL(zero_u64_kernel, dim3((unsigned)max((int64_t)1, min((int64_t)1024, (cells + 255) / 256))),
+                           dim3(256), 0, s, a.counters, cells, (uint32_t*)nullptr);
+        const int64_t grid = traverse_grid(a, y);
+        if (y.lds_counters) {
+            hipLaunchKernelGGL(traverse_kernel<true>, dim3((unsigned)grid), dim3(kWave), y.lds_bytes, s, a, y);
+        } else {
+            if (!a.gscratch) return fail(-1, "query: counter scratch missing");
+            hipLaunchKernelGGL(traverse_kernel<false>, dim3((unsigned)grid), dim3(kWave), y.lds_bytes, s, a, y);
+        }
+        DCIH_HIP(hipGetLastError());
+        rc = rank_rows(ws_rank, chunk, a.nq, a.N, a_in.k, true, a_in.out_ids + (int64_t)q0 * a_in.k,
+                       a_in.out_dists ? a_in.out_dists + (int64_t)q0 * a_in.k : nullptr, s);
+        if (rc) return rc;
+    }
     return 0;
 }
 

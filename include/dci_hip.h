@@ -126,14 +126,15 @@ int dcih_append(dcih_index* h, int dim, int64_t num_points, const float* d_data,
  *
  * num_neighbours may be as large as the number of indexed points (what
  * dciknn_cuda/core.py:84-85 passes when the caller gives none).  Up to 8192 the
- * traversal keeps its best candidates in on-chip tables.  Above 8192 it must also
- * exceed the points per partition, ceil(num_points / block_size): the stop rule
- * (:598-607) counts promotions of one partition, so it can then never fire, every
- * point is promoted, and the result, the num_neighbours closest of all points by
- * (distance, id), is computed directly (all distances, one sort per query; the
- * counters from their closed forms).  Distances on this path are summed in index
- * order like compute_dist_device (:36-44).  8192 < num_neighbours <= points per
- * partition returns DCIH_EUNSUPPORTED (equality is accepted without d_counters).
+ * traversal keeps its best candidates in on-chip tables.  Above 8192 and above the
+ * points per partition, ceil(num_points / block_size), the stop rule (:598-607),
+ * which counts promotions of one partition, can never fire: every point is
+ * promoted, and the result, the num_neighbours closest of all points by (distance,
+ * id), is computed directly (all distances, summed in index order like
+ * compute_dist_device, :36-44; one sort per query; the counters from their closed
+ * forms).  Above 8192 otherwise, the traversal records every candidate's distance
+ * in a row of num_points cells per query and the rows are sorted; both paths work
+ * through the queries in chunks and use up to 2 GB of workspace.
  *
  * blind != 0 (query_config.blind, :498-505, :754-773, :859-864): the same
  * traversal under the same stop rule, but no distance is computed.  d_nn is
@@ -145,7 +146,8 @@ int dcih_append(dcih_index* h, int dim, int64_t num_points, const float* d_data,
  * step numbers as floats (+inf beside -1).  The reference ranks blind
  * candidates by a count that is 1 for every one of them and collects them
  * through per-thread cursors that overwrite each other, so it defines no order;
- * this one does.  R above 8192 returns DCIH_EUNSUPPORTED.
+ * this one does.  R above 8192 takes the row-per-query path described above and
+ * needs step numbers below 2^24 (else DCIH_EUNSUPPORTED).
  */
 int dcih_query(dcih_index* h, int dim, int num_queries, const float* d_query,
                int num_neighbours, int blind, int num_outer_iterations,

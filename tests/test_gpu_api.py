@@ -248,11 +248,17 @@ def test_full_ranking_through_the_binding(gpu, B):
     dci.free()
 
 
-def test_large_k_below_partition_size_is_refused(gpu):
-    rng = np.random.default_rng(13)
-    X = torch.from_numpy(rng.standard_normal((20000, 8)).astype(np.float32)).cuda()
-    dci = gpu.DCI(8, 2, 3, 2, 4, seed=2)      # 10000 points per partition
-    dci.add(X)
-    with pytest.raises(RuntimeError):
-        dci.query(X[:1], 9000)
-    dci.free()
+@pytest.mark.parametrize("n,B,T,k,outer", [(20000, 2, 1, 9000, 50),     # partitions stop once 9000 of their 10000 points are promoted
+                                           (30000, 2, 2, 8200, 100000),  # lane-0 promotions never reach k: runs dry
+                                           (9000, 1, 1, -1, 50)])        # k = N = points per partition, with counters
+def test_large_k_with_early_stops(gpu, oracle, n, B, T, k, outer):
+    """num_neighbours above 8192 but not above the points per partition: the stop rule can
+    fire, so the traversal runs (step-by-step kernel, every candidate recorded in a dense
+    row per query) and the rows are sorted.  Counters exact, neighbours as in the oracle."""
+    ids, dists, ctr, ref, X, Q = _full_ranking_case(gpu, oracle, n, 3, 12, 2, 3, B, T, k, outer=outer)
+    np.testing.assert_array_equal(ctr, ref["counters"].astype(np.int64))
+    assert set_agreement_rows(ids, ref["ids"]) >= 0.999
+    np.testing.assert_array_equal(ids < 0, ref["ids"] < 0)
+    np.testing.assert_allclose(dists, ref["dists"], rtol=1e-5)
+    if B == 2 and T == 1:
+        assert np.all(ctr[:, 1] < n), "the case is meant to stop before everything is promoted"

@@ -134,10 +134,17 @@ def test_blind_python_surface(gpu, oracle):
     mdci.free()
 
 
-def test_blind_rejects_too_many_slots(gpu):
-    X, Q = _data(2, 20000, 2, 8)
-    dci = gpu.DCI(8, 2, 3, 2, 4, seed=1)
+def test_blind_more_than_8192_slots(gpu, oracle):
+    """min(10k, outer) above the top-k tables: candidates are recorded in a dense row
+    per query and sorted from there; same ids, steps and counters as the oracle."""
+    n, dim, M, L, B, T, k, outer = 30000, 8, 2, 3, 2, 4, 1000, 9000      # 9000 slots
+    X, Q = _data(2, n, 3, dim)
+    dci = gpu.DCI(dim, M, L, B, T, seed=1)
     dci.add(torch.from_numpy(X).cuda())
-    with pytest.raises(RuntimeError):
-        dci.query(torch.from_numpy(Q).cuda(), 1000, 9000, blind=True)     # min(10000, 9000) > 8192
+    ids, steps, ctr = _engine_blind(dci, torch.from_numpy(Q).cuda(), k, outer, 10 * k, B, T)
+    skeys, sids = engine_index(dci)
+    qproj = engine_project(dci.directions.numpy(), Q).T.copy()
+    ref = oracle.query_blind(skeys, sids, qproj, M, L, B, T, k, outer, max_cand=10 * k)
     dci.free()
+    assert ids.shape == (3, 9000)
+    _check(ids, steps, ctr, ref, visits=True)
