@@ -6,11 +6,11 @@
 // block_size*thread_size threads quicksorts whole slices serially.
 //
 // Here a (key, position-in-slice) pair is one 64-bit word whose unsigned order
-// is the wanted order, so a slice of up to kTileCap points is sorted by one
+// is the wanted order.  A slice of up to 32256 points is sorted by one
 // workgroup entirely in LDS: one coalesced read of the keys, one coalesced
 // write of the sorted keys and ids.  Longer slices are sorted tile by tile and
-// the tiles are then merged pairwise in global memory (merge path), each pass
-// doubling the run length.
+// the tiles are then merged pairwise (merge path, staged through LDS), each
+// pass doubling the run length, the last one writing the final arrays.
 #include "common.h"
 #include "kernels.h"
 
@@ -26,6 +26,7 @@ struct SegGeom {
     int64_t ppb;      // points per partition
     int B;            // partitions
     int tiles;        // tiles per partition (by the longest partition)
+    int tile_size;    // points per tile
 };
 
 __device__ inline unsigned long long pack_key(float key, uint32_t pos) {
@@ -107,12 +108,14 @@ __global__ void segsort_tile_kernel(const float* __restrict__ keys, SegGeom g,
 // inverse written once, all coalesced.
 constexpr int kRadixMax = 63 * 512;
 constexpr int kRadixMin = 512;        // up to this the bitonic tile kernel is faster
+constexpr int kRadixTile = 30 * 1024; // longest tile of a slice that needs merge passes
 
 template <int kRadixThreads, int IPT>
 // (256 threads with more than 45 items each: registers for two workgroups per CU)
 __global__ __launch_bounds__(kRadixThreads, (kRadixThreads == 256 && IPT > 45) ? 2 : 1) void segsort_radix_kernel(
     const float* __restrict__ keys, SegGeom g, float* __restrict__ skeys,
-    int32_t* __restrict__ sids, uint32_t* __restrict__ inv, uint16_t* __restrict__ lids) {
+    int32_t* __restrict__ sids, uint32_t* __restrict__ inv, uint16_t* __restrict__ lids,
+    unsigned long long* __restrict__ packed) {
     extern __shared__ uint32_t rs[];
     uint32_t* stage = rs;                                         // IPT*1024 words
     uint16_t* stage16 = reinterpret_cast<uint16_t*>(rs);
@@ -122,12 +125,19 @@ __global__ __launch_bounds__(kRadixThreads, (kRadixThreads == 256 && IPT > 45) ?
 
     const int tid = threadIdx.x;
     const int lane = tid & 63, wave = tid >> 6;
-    const int b = (int)(blockIdx.x % g.B);
-    const int64_t i = blockIdx.x / g.B;
+    // packed == null: the workgroup sorts a whole slice and writes the final arrays;
+    // else it sorts one tile of a slice into packed (key, position in slice) words
+    // for the merge passes
+    const int tiles = packed ? g.tiles : 1;
+    const int tile = (int)(blockIdx.x % tiles);
+    const int b = (int)((blockIdx.x / tiles) % g.B);
+    const int64_t i = blockIdx.x / ((int64_t)tiles * g.B);
     const int64_t off = (int64_t)b * g.ppb;
-    const int n = (int)min(g.n - off, g.ppb);
+    const int64_t t0 = packed ? (int64_t)tile * g.tile_size : 0;
+    const int64_t nseg = min(g.n - off, g.ppb) - t0;
+    const int n = (int)(packed ? min(nseg, (int64_t)g.tile_size) : nseg);
     if (n <= 0) return;
-    const int64_t base = i * g.n + off;
+    const int64_t base = i * g.n + off + t0;
 
     if (tid < 2) misc[32 + tid] = tid ? 0xffffffffu : 0u;        // OR / AND of all keys
     uint32_t k[IPT], rp[IPT];      // rp: id in the low half, rank / position in the high half
@@ -244,6 +254,26 @@ __global__ __launch_bounds__(kRadixThreads, (kRadixThreads == 256 && IPT > 45) ?
         }
     }
 
+    if (packed) {      // (same on every thread) keys, then ids, through LDS into coalesced order
+        __syncthreads();
+#pragma unroll
+        for (int r = 0; r < IPT; r++) stage[tid * IPT + r] = k[r];
+        __syncthreads();
+#pragma unroll
+        for (int r = 0; r < IPT; r++) k[r] = stage[r * kRadixThreads + tid];
+        __syncthreads();
+#pragma unroll
+        for (int r = 0; r < IPT; r++) stage[tid * IPT + r] = rp[r] & 0xffffu;
+        __syncthreads();
+#pragma unroll
+        for (int r = 0; r < IPT; r++) {
+            const int j = r * kRadixThreads + tid;
+            if (j < n)
+                packed[base + j] = ((unsigned long long)k[r] << 32) | (uint32_t)(t0 + stage[j]);
+        }
+        return;
+    }
+
     // results, through LDS so that every global write is coalesced
     __syncthreads();
 #pragma unroll
@@ -270,7 +300,8 @@ __global__ __launch_bounds__(kRadixThreads, (kRadixThreads == 256 && IPT > 45) ?
 
 template <int NT, int IPT>
 static int launch_radix(const float* d_keys, const SegGeom& g, int num_indices, float* d_skeys,
-                        int32_t* d_sids, uint32_t* d_inv, uint16_t* d_lids, hipStream_t s) {
+                        int32_t* d_sids, uint32_t* d_inv, uint16_t* d_lids,
+                        unsigned long long* d_packed, hipStream_t s) {
     const size_t lds = (size_t)(IPT * NT + 8 * NT + 64) * sizeof(uint32_t);
     static bool attr_done = false;
     if (!attr_done) {
@@ -278,18 +309,50 @@ static int launch_radix(const float* d_keys, const SegGeom& g, int num_indices, 
                                      hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds));
         attr_done = true;
     }
-    const int64_t blocks = (int64_t)num_indices * g.B;
+    const int64_t blocks = (int64_t)num_indices * g.B * (d_packed ? g.tiles : 1);
+    if (blocks > 0x7fffffffLL) return fail(-1, "segsort: too many slices for one launch");
     hipLaunchKernelGGL((segsort_radix_kernel<NT, IPT>), dim3((unsigned)blocks), dim3(NT), lds, s,
-                       d_keys, g, d_skeys, d_sids, d_inv, d_lids);
+                       d_keys, g, d_skeys, d_sids, d_inv, d_lids, d_packed);
     DCIH_HIP(hipGetLastError());
     return 0;
 }
 
+// Merge path: how many elements of A are among the first d outputs of merging A
+// (la elements) with B (lb elements), A winning ties (its positions are smaller).
+// One wavefront searches 64 split points per round.
+__device__ inline int64_t merge_split_wave(const unsigned long long* __restrict__ A, int64_t la,
+                                           const unsigned long long* __restrict__ Bv, int64_t lb,
+                                           int64_t d, int lane) {
+    int64_t lo = max((int64_t)0, d - lb), hi = min(d, la);
+    while (lo < hi) {       // smallest a in [lo, hi] with !(A[a] < B[d-1-a]); wave-uniform
+        const int64_t step = (hi - lo + kWave - 1) / kWave;
+        const int64_t a = lo + (int64_t)lane * step;
+        const bool valid = a < hi;
+        const bool below = valid && A[a] < Bv[d - 1 - a];
+        const int t = __popcll(__ballot(below));      // the predicate is monotone: a prefix of lanes
+        if (t == 0) { hi = lo; break; }
+        const int64_t new_lo = lo + (int64_t)(t - 1) * step + 1;
+        hi = min(hi, lo + (int64_t)t * step);
+        lo = new_lo;
+    }
+    return lo;
+}
+
 // One merge pass: within every slice, neighbouring sorted runs of length `run`
-// are merged into runs of 2*run.  A workgroup produces kMergeChunk outputs.
+// (a multiple of kMergeChunk / 2) are merged into runs of 2*run.  A workgroup
+// produces kMergeChunk outputs: two wavefronts find where its piece starts and
+// ends in either run, the two pieces are read into LDS with coalesced loads,
+// every thread merges kMergeItems outputs there, and the outputs leave in
+// coalesced stores.  The last pass (skeys != null) writes the final arrays
+// instead of packed words.
 __global__ __launch_bounds__(kMergeThreads) void segsort_merge_kernel(
     const unsigned long long* __restrict__ src, unsigned long long* __restrict__ dst,
-    SegGeom g, int chunks, int64_t run) {
+    SegGeom g, int chunks, int64_t run, float* __restrict__ skeys, int32_t* __restrict__ sids,
+    uint32_t* __restrict__ inv, uint16_t* __restrict__ lids) {
+    __shared__ unsigned long long s_in[kMergeChunk];
+    __shared__ unsigned long long s_out[kMergeChunk];
+    __shared__ int64_t s_split[2];
+    const int tid = threadIdx.x, lane = tid & (kWave - 1), wave = tid / kWave;
     const int64_t flat = blockIdx.x;
     const int chunk = (int)(flat % chunks);
     const int b = (int)((flat / chunks) % g.B);
@@ -306,40 +369,54 @@ __global__ __launch_bounds__(kMergeThreads) void segsort_merge_kernel(
     const int64_t la = a1 - a0, lb = b1 - b0;
     const unsigned long long* A = src + base + a0;
     const unsigned long long* Bv = src + base + b0;
-
-    int64_t d = o0 - ps + (int64_t)threadIdx.x * kMergeItems;   // first output of this thread
-    if (d >= la + lb) return;
-    // merge path: number of A elements among the first d outputs
-    int64_t lo = max((int64_t)0, d - lb), hi = min(d, la);
-    while (lo < hi) {
-        const int64_t a = (lo + hi) >> 1;
-        if (A[a] < Bv[d - 1 - a]) lo = a + 1; else hi = a;
+    const int64_t d0 = o0 - ps;                               // first output of this workgroup
+    const int64_t d1 = min(d0 + kMergeChunk, la + lb);
+    const int cnt = (int)(d1 - d0);
+    if (wave < 2) {
+        const int64_t sp = merge_split_wave(A, la, Bv, lb, wave ? d1 : d0, lane);
+        if (lane == 0) s_split[wave] = sp;
     }
-    int64_t ia = lo, ib = d - lo;
-    unsigned long long* out = dst + base + ps + d;
-    const int cnt = (int)min((int64_t)kMergeItems, la + lb - d);
-    unsigned long long va = ia < la ? A[ia] : ~0ull;
-    unsigned long long vb = ib < lb ? Bv[ib] : ~0ull;
-    for (int t = 0; t < cnt; t++) {
-        const bool takeA = ib >= lb || (ia < la && va < vb);
-        if (takeA) { out[t] = va; ia++; va = ia < la ? A[ia] : ~0ull; }
-        else       { out[t] = vb; ib++; vb = ib < lb ? Bv[ib] : ~0ull; }
+    __syncthreads();
+    const int64_t ia0 = s_split[0], ia1 = s_split[1];
+    const int64_t ib0 = d0 - ia0;
+    const int na = (int)(ia1 - ia0), nb = cnt - na;
+    for (int j = tid; j < cnt; j += kMergeThreads)
+        s_in[j] = j < na ? A[ia0 + j] : Bv[ib0 + (j - na)];
+    __syncthreads();
+    {
+        const unsigned long long* LA = s_in;
+        const unsigned long long* LB = s_in + na;
+        const int d = tid * kMergeItems;
+        if (d < cnt) {
+            int lo = max(0, d - nb), hi = min(d, na);
+            while (lo < hi) {
+                const int a = (lo + hi) >> 1;
+                if (LA[a] < LB[d - 1 - a]) lo = a + 1; else hi = a;
+            }
+            int ia = lo, ib = d - lo;
+            const int m = min(kMergeItems, cnt - d);
+            unsigned long long va = ia < na ? LA[ia] : ~0ull;
+            unsigned long long vb = ib < nb ? LB[ib] : ~0ull;
+            for (int t = 0; t < m; t++) {
+                const bool takeA = ib >= nb || (ia < na && va < vb);
+                if (takeA) { s_out[d + t] = va; ia++; va = ia < na ? LA[ia] : ~0ull; }
+                else       { s_out[d + t] = vb; ib++; vb = ib < nb ? LB[ib] : ~0ull; }
+            }
+        }
     }
-}
-
-__global__ void segsort_unpack_kernel(const unsigned long long* __restrict__ packed,
-                                      int64_t total, int64_t n, int64_t ppb,
-                                      float* __restrict__ skeys, int32_t* __restrict__ sids,
-                                      uint32_t* __restrict__ inv, uint16_t* __restrict__ lids) {
-    const int64_t stride = (int64_t)gridDim.x * blockDim.x;
-    for (int64_t e = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; e < total; e += stride) {
-        const unsigned long long w = packed[e];
-        const int64_t col = e % n;
-        const int64_t off = (col / ppb) * ppb;
-        skeys[e] = ord2f((uint32_t)(w >> 32));
-        sids[e] = (int32_t)(off + (uint32_t)w);
-        if (inv) inv[e - col + off + (uint32_t)w] = (uint32_t)(col - off);
-        if (lids) lids[e] = (uint16_t)(uint32_t)w;
+    __syncthreads();
+    const int64_t out0 = base + ps + d0;
+    if (!skeys) {
+        for (int j = tid; j < cnt; j += kMergeThreads) dst[out0 + j] = s_out[j];
+    } else {
+        for (int j = tid; j < cnt; j += kMergeThreads) {
+            const unsigned long long w = s_out[j];
+            const int64_t e = out0 + j;
+            skeys[e] = ord2f((uint32_t)(w >> 32));
+            sids[e] = (int32_t)(off + (uint32_t)w);
+            if (inv) inv[base + (uint32_t)w] = (uint32_t)(ps + d0 + j);
+            if (lids) lids[e] = (uint16_t)(uint32_t)w;
+        }
     }
 }
 
@@ -364,6 +441,7 @@ int segsort(const float* d_keys, int num_indices, int64_t n, int block_size,
     g.B = block_size;
     g.ppb = (n + block_size - 1) / block_size;
     g.tiles = (int)((g.ppb + kTileCap - 1) / kTileCap);
+    g.tile_size = kTileCap;
     const int np2 = next_pow2((int)min((int64_t)kTileCap, g.ppb));
     // at most kTileCap / 1024 elements per thread (the inverse-permutation pass relies on it)
     const int threads = max(64, min(1024, np2 / 2));
@@ -376,9 +454,6 @@ int segsort(const float* d_keys, int num_indices, int64_t n, int block_size,
         DCIH_HIP(hipFuncSetAttribute((const void*)segsort_tile_kernel<true>,
                                      hipFuncAttributeMaxDynamicSharedMemorySize,
                                      kTileCap * (int)sizeof(unsigned long long)));
-        DCIH_HIP(hipFuncSetAttribute((const void*)segsort_tile_kernel<false>,
-                                     hipFuncAttributeMaxDynamicSharedMemorySize,
-                                     kTileCap * (int)sizeof(unsigned long long)));
         attr_done[0] = true;
     }
 
@@ -386,7 +461,7 @@ int segsort(const float* d_keys, int num_indices, int64_t n, int block_size,
         // odd items-per-thread keep the blocked LDS accesses free of bank conflicts
 #define DCIH_RADIX(NT, IPT) \
     if (g.ppb <= (int64_t)(NT) * (IPT))  \
-        return launch_radix<NT, IPT>(d_keys, g, num_indices, d_skeys, d_sids, d_inv, d_lids, s)
+        return launch_radix<NT, IPT>(d_keys, g, num_indices, d_skeys, d_sids, d_inv, d_lids, nullptr, s)
         DCIH_RADIX(64, 9); DCIH_RADIX(64, 17); DCIH_RADIX(64, 25); DCIH_RADIX(64, 33);
         DCIH_RADIX(128, 21); DCIH_RADIX(128, 27); DCIH_RADIX(128, 33);
         DCIH_RADIX(256, 21); DCIH_RADIX(256, 27); DCIH_RADIX(256, 33); DCIH_RADIX(256, 39); DCIH_RADIX(256, 45);
@@ -404,20 +479,30 @@ int segsort(const float* d_keys, int num_indices, int64_t n, int block_size,
     if (!d_tmp) return fail(-1, "segsort: scratch buffer missing");
     unsigned long long* bufA = (unsigned long long*)d_tmp;
     unsigned long long* bufB = bufA + (size_t)num_indices * n;
-    hipLaunchKernelGGL(segsort_tile_kernel<false>, dim3((unsigned)blocks), dim3(threads), lds, s,
-                       d_keys, g, (float*)nullptr, (int32_t*)nullptr, (uint32_t*)nullptr, (uint16_t*)nullptr, bufA, np2);
+    // Slices beyond one LDS pass: as few radix-sorted tiles as cover the slice (runs of a
+    // multiple of 1024 points, so that a merge chunk never straddles two pairs of runs),
+    // then merge passes.
+    g.tiles = (int)((g.ppb + kRadixTile - 1) / kRadixTile);
+    g.tile_size = (int)((((g.ppb + g.tiles - 1) / g.tiles) + 1023) / 1024 * 1024);
+    {
+        int rc = -1;
+#define DCIH_RADIX_TILE(NT, IPT) \
+    if (rc < 0 && g.tile_size <= (NT) * (IPT))  \
+        rc = launch_radix<NT, IPT>(d_keys, g, num_indices, nullptr, nullptr, nullptr, nullptr, bufA, s)
+        DCIH_RADIX_TILE(512, 33); DCIH_RADIX_TILE(512, 39); DCIH_RADIX_TILE(512, 45);
+        DCIH_RADIX_TILE(512, 51); DCIH_RADIX_TILE(512, 57); DCIH_RADIX_TILE(512, 63);
+#undef DCIH_RADIX_TILE
+        if (rc) return rc < 0 ? fail(-1, "segsort: no radix configuration for the tile size") : rc;
+    }
     const int chunks = (int)((g.ppb + kMergeChunk - 1) / kMergeChunk);
     const int64_t mblocks = (int64_t)num_indices * g.B * chunks;
     if (mblocks > 0x7fffffffLL) return fail(-1, "segsort: too many merge chunks for one launch");
-    for (int64_t run = kTileCap; run < g.ppb; run *= 2) {
+    for (int64_t run = g.tile_size; run < g.ppb; run *= 2) {
+        const bool last = run * 2 >= g.ppb;       // the last pass writes the final arrays
         hipLaunchKernelGGL(segsort_merge_kernel, dim3((unsigned)mblocks), dim3(kMergeThreads), 0, s,
-                           bufA, bufB, g, chunks, run);
+                           bufA, bufB, g, chunks, run, last ? d_skeys : (float*)nullptr, d_sids, d_inv, d_lids);
         unsigned long long* t = bufA; bufA = bufB; bufB = t;
     }
-    const int64_t total = (int64_t)num_indices * n;
-    const int ublocks = (int)min((int64_t)65536, (total + 255) / 256);
-    hipLaunchKernelGGL(segsort_unpack_kernel, dim3(ublocks), dim3(256), 0, s,
-                       bufA, total, n, g.ppb, d_skeys, d_sids, d_inv, d_lids);
     DCIH_HIP(hipGetLastError());
     return 0;
 }

@@ -249,7 +249,6 @@ __global__ __launch_bounds__(NT, MINW) void traverse_block_kernel(QueryArgs a, B
     };
     const int I = a.M * a.L;
     const int S = 2 * I;                       // streams
-    const uint32_t Lm1 = (uint32_t)a.L - 1u;
 
     // Workgroups go to the XCDs round-robin by their number, and every XCD has an L2
     // of its own.  XCD x gets the partitions x, x + 8, ... and works through them one
@@ -340,25 +339,6 @@ __global__ __launch_bounds__(NT, MINW) void traverse_block_kernel(QueryArgs a, B
         st.key = a.skeys + (int64_t)i * a.N + off;
         st.n = n; st.T = T; st.p = s_p[i]; st.side = s & 1; st.q = s_qp[i];
         return st;
-    };
-    // count_below over the epoch's range [cprev, c) of stream sidx, narrowed first by
-    // the 15 priorities sampled from that range (LDS), then by key reads
-    auto count_in_epoch = [&](int sidx, uint32_t x, bool strict) {
-        int lo = s_cprev[sidx], hi = s_c[sidx];
-        const int len = hi - lo;
-        if (len >= 32) {
-            const uint32_t* tab = s_samp + sidx * 16;
-            int tl = 0, th = 15;            // number of samples t in 1..15 below x (monotone)
-            while (tl < th) {
-                const int mid = (tl + th + 1) >> 1;
-                const uint32_t v = tab[mid];
-                if (strict ? v < x : v <= x) tl = mid; else th = mid - 1;
-            }
-            const int base0 = lo;
-            if (tl > 0) lo = base0 + (int)(((int64_t)len * tl) >> 4) + 1;
-            if (tl < 15) hi = base0 + (int)(((int64_t)len * (tl + 1)) >> 4);
-        }
-        return count_below(load_stream(sidx), x, strict, lo, hi, probes);
     };
 
     // Adds (or, for undo, removes) the visits of windows [cprev, c) of all streams.
