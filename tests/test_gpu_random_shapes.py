@@ -1,7 +1,8 @@
 """Randomised traversal parity: both query kernels against the CPU oracle on many
 small seeded shapes, including the awkward corners (L = 1, where every visit is a
 promotion; duplicated points, where priorities tie everywhere; windows wider
-than a partition; budgets of 0 and 1 iterations; tiny max_num_candidates)."""
+than a partition; budgets of 0 and 1 iterations; tiny max_num_candidates),
+each shape queried with distances and blind."""
 import os
 
 import numpy as np
@@ -58,7 +59,7 @@ def test_random_shape(gpu, oracle, seed):
         k = int(rng.choice([1, 10, 40]))
     X, Q = _points(rng, n, nq, dim, kind)
     xd, qd = torch.from_numpy(X).cuda(), torch.from_numpy(Q).cuda()
-    ref = None
+    ref = bref = None
     for traversal in ("step", "auto"):
         dci = gpu.DCI(dim, M, L, B, T, seed=seed, traversal=traversal)
         dci.add(xd)
@@ -73,6 +74,22 @@ def test_random_shape(gpu, oracle, seed):
             skeys, sids = engine_index(dci)
             qproj = engine_project(dci.directions.numpy(), Q).T.copy()
             ref = oracle.query(skeys, sids, X, Q, qproj, M, L, B, T, k, outer, max_cand=max_cand)
+        # blind querying of the same shape: integer work, so ids and steps match exactly
+        R = min(max_cand, outer)
+        if R >= 1:
+            bids = torch.full((nq, R), -7, dtype=torch.int32, device="cuda")
+            bsteps = torch.full((nq, R), -7.0, dtype=torch.float32, device="cuda")
+            _capi.check(dci._lib.dcih_query(dci._dci_inst, dim, nq, qd.data_ptr(), k, 1, outer, max_cand,
+                                            B, T, bids.data_ptr(), bsteps.data_ptr(), None,
+                                            torch.cuda.current_stream().cuda_stream))
+            torch.cuda.synchronize()
+            if bref is None:
+                bref = oracle.query_blind(skeys, sids, qproj, M, L, B, T, k, outer, max_cand=max_cand)
+            np.testing.assert_array_equal(bids.cpu().numpy(), bref["ids"], err_msg="blind ids " + traversal)
+            want = bref["steps"].astype(np.float64)
+            want[bref["ids"] < 0] = np.inf
+            np.testing.assert_array_equal(bsteps.cpu().numpy().astype(np.float64), want,
+                                          err_msg="blind steps " + traversal)
         dci.free()
         tag = "%s %s" % (traversal, (M, L, n, B, T, k, outer, max_cand, dim, kind))
         ids, dists, ctr = ids.cpu().numpy(), dists.cpu().numpy(), ctr.cpu().numpy()
