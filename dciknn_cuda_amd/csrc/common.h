@@ -4,6 +4,7 @@
 #include <hip/hip_runtime.h>
 #include <stdint.h>
 
+#include <mutex>
 #include <string>
 
 namespace dcih {
@@ -19,6 +20,26 @@ int fail(int code, const std::string& msg);
         if (e_ != hipSuccess)                                                   \
             return ::dcih::fail(-3, std::string(#call) + ": " + hipGetErrorString(e_)); \
     } while (0)
+
+// Runs `set_up` once per device (the current one) and remembers success: kernel
+// attributes are kept per device, and several host threads may launch at once.
+class DeviceOnce {
+public:
+    template <class F>
+    int run(F set_up) {
+        int dev = 0;
+        if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= kMaxDevices) return set_up();
+        std::lock_guard<std::mutex> lock(mu_);
+        if (done_[dev]) return 0;
+        const int rc = set_up();
+        if (rc == 0) done_[dev] = true;
+        return rc;
+    }
+private:
+    static constexpr int kMaxDevices = 64;
+    std::mutex mu_;
+    bool done_[kMaxDevices] = {};
+};
 
 // ---- order-preserving float <-> uint32 ------------------------------------
 // Ascending unsigned order of the result equals ascending float order

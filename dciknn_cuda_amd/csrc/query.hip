@@ -320,6 +320,20 @@ int merge_cap(int k) {
 
 }  // namespace
 
+// The traversal and merge kernels may use all of a CU's LDS.
+static int allow_full_lds() {
+    static DeviceOnce once;
+    return once.run([]() -> int {
+        DCIH_HIP(hipFuncSetAttribute((const void*)traverse_kernel<true>,
+                                     hipFuncAttributeMaxDynamicSharedMemorySize, kMaxLds));
+        DCIH_HIP(hipFuncSetAttribute((const void*)traverse_kernel<false>,
+                                     hipFuncAttributeMaxDynamicSharedMemorySize, kMaxLds));
+        DCIH_HIP(hipFuncSetAttribute((const void*)merge_topk_kernel,
+                                     hipFuncAttributeMaxDynamicSharedMemorySize, kMaxLds));
+        return 0;
+    });
+}
+
 size_t query_part_bytes(const QueryArgs& a) {
     return (size_t)a.nq * a.B * a.kcap * sizeof(unsigned long long);
 }
@@ -353,15 +367,9 @@ int query(const QueryArgs& a_in, hipStream_t s, hipEvent_t* ev) {
     if (a.mode == 2 && !can_block)
         return fail(-4, "query: this shape does not fit the batch traversal kernel");
     const bool use_block = a.mode != 1 && can_block;
-    static bool attr_done = false;
-    if (!attr_done) {
-        DCIH_HIP(hipFuncSetAttribute((const void*)traverse_kernel<true>,
-                                     hipFuncAttributeMaxDynamicSharedMemorySize, kMaxLds));
-        DCIH_HIP(hipFuncSetAttribute((const void*)traverse_kernel<false>,
-                                     hipFuncAttributeMaxDynamicSharedMemorySize, kMaxLds));
-        DCIH_HIP(hipFuncSetAttribute((const void*)merge_topk_kernel,
-                                     hipFuncAttributeMaxDynamicSharedMemorySize, kMaxLds));
-        attr_done = true;
+    {
+        const int rc = allow_full_lds();
+        if (rc) return rc;
     }
     {   // zero the counters and the redo count with a kernel (safe under graph capture)
         const int64_t cells = a.counters ? (int64_t)a.nq * 4 : 0;
@@ -406,13 +414,9 @@ int query_dense(const QueryArgs& a_in, const float* d_dirs, void* ws, int chunk,
     // blind scores are step numbers stored as floats: they must stay exact
     if (a_in.blind && (int64_t)a_in.L * (a_in.ppb + 2 * (int64_t)a_in.T) >= (1 << 24))
         return fail(-4, "query: this many blind results need step numbers below 2^24; use a larger block_size");
-    static bool attr_done = false;
-    if (!attr_done) {
-        DCIH_HIP(hipFuncSetAttribute((const void*)traverse_kernel<true>,
-                                     hipFuncAttributeMaxDynamicSharedMemorySize, kMaxLds));
-        DCIH_HIP(hipFuncSetAttribute((const void*)traverse_kernel<false>,
-                                     hipFuncAttributeMaxDynamicSharedMemorySize, kMaxLds));
-        attr_done = true;
+    {
+        const int rc = allow_full_lds();
+        if (rc) return rc;
     }
     const size_t qp_bytes = ((size_t)I * chunk * sizeof(float) + 255) & ~(size_t)255;
     float* d_qproj = (float*)ws;

@@ -303,11 +303,14 @@ static int launch_radix(const float* d_keys, const SegGeom& g, int num_indices, 
                         int32_t* d_sids, uint32_t* d_inv, uint16_t* d_lids,
                         unsigned long long* d_packed, hipStream_t s) {
     const size_t lds = (size_t)(IPT * NT + 8 * NT + 64) * sizeof(uint32_t);
-    static bool attr_done = false;
-    if (!attr_done) {
-        DCIH_HIP(hipFuncSetAttribute((const void*)segsort_radix_kernel<NT, IPT>,
-                                     hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds));
-        attr_done = true;
+    static DeviceOnce once;
+    {
+        const int rc = once.run([lds]() -> int {
+            DCIH_HIP(hipFuncSetAttribute((const void*)segsort_radix_kernel<NT, IPT>,
+                                         hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds));
+            return 0;
+        });
+        if (rc) return rc;
     }
     const int64_t blocks = (int64_t)num_indices * g.B * (d_packed ? g.tiles : 1);
     if (blocks > 0x7fffffffLL) return fail(-1, "segsort: too many slices for one launch");
@@ -449,12 +452,15 @@ int segsort(const float* d_keys, int num_indices, int64_t n, int block_size,
     const int64_t blocks = (int64_t)num_indices * g.B * g.tiles;
     if (blocks > 0x7fffffffLL) return fail(-1, "segsort: too many slices for one launch");
 
-    static bool attr_done[2] = {false, false};
-    if (!attr_done[0]) {
-        DCIH_HIP(hipFuncSetAttribute((const void*)segsort_tile_kernel<true>,
-                                     hipFuncAttributeMaxDynamicSharedMemorySize,
-                                     kTileCap * (int)sizeof(unsigned long long)));
-        attr_done[0] = true;
+    static DeviceOnce once;
+    {
+        const int rc = once.run([]() -> int {
+            DCIH_HIP(hipFuncSetAttribute((const void*)segsort_tile_kernel<true>,
+                                         hipFuncAttributeMaxDynamicSharedMemorySize,
+                                         kTileCap * (int)sizeof(unsigned long long)));
+            return 0;
+        });
+        if (rc) return rc;
     }
 
     if (g.ppb > kRadixMin && g.ppb <= kRadixMax) {

@@ -1067,12 +1067,13 @@ int query_block(const QueryArgs& a, hipStream_t s) {
     const int fit = (int)(160 * 1024 / y.lds_bytes);      // workgroups per CU by LDS
 #define DCIH_LAUNCH(CB, MW)                                                                        \
     do {                                                                                           \
-        static bool attr_done = false;                                                             \
-        if (!attr_done) {                                                                          \
+        static DeviceOnce once;                                                                    \
+        const int rc_attr = once.run([]() -> int {                                                 \
             DCIH_HIP(hipFuncSetAttribute((const void*)traverse_block_kernel<kBlockThreads, CB, MW>, \
                                          hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024)); \
-            attr_done = true;                                                                      \
-        }                                                                                          \
+            return 0;                                                                              \
+        });                                                                                        \
+        if (rc_attr) return rc_attr;                                                               \
         hipLaunchKernelGGL((traverse_block_kernel<kBlockThreads, CB, MW>), dim3((unsigned)items),  \
                            dim3(kBlockThreads), y.lds_bytes, s, a, y);                             \
     } while (0)
