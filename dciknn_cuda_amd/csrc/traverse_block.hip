@@ -307,10 +307,11 @@ __global__ __launch_bounds__(NT, MINW) void traverse_block_kernel(QueryArgs a, B
     // waiting.  The total doubles from epoch to epoch until one has to be undone.
     // hint = running average of the step at which earlier queries stopped in this
     // partition; it only steers epoch sizes, never results.  The first jump aims
-    // 5 % past it.  The number of points whose counters are complete grows like a
+    // 12 % past it.  The number of points whose counters are complete grows like a
     // high power (L) of the steps taken, so stop steps of one partition scatter
-    // little and most items finish in one or two epochs, while a jump 20 % too far
-    // already brings several times the promotions needed and overflows the tables.
+    // little and most items finish in one epoch (12 % more steps bring about three
+    // times the promotions to rank, which still costs less than a second epoch),
+    // while a jump much farther overflows the tables.
     // Where the stop needs more promotions than one epoch may produce (their
     // number at earlier stops in this partition is the second hint; about k * T
     // without one), the jump is shortened by the same power law so that an epoch
@@ -320,7 +321,7 @@ __global__ __launch_bounds__(NT, MINW) void traverse_block_kernel(QueryArgs a, B
     const float inv_L = 1.0f / (float)a.L;
     const float hint = a.stop_hint ? a.stop_hint[b] : 0.0f;
     const float hint_promos = a.stop_hint ? a.stop_hint[a.B + b] : 0.0f;
-    const float kHintFirst = fminf(1.05f,
+    const float kHintFirst = fminf(1.12f,
         fast_pow(kPromoAim / fmaxf(1.0f, hint_promos > 0.0f ? hint_promos : (float)a.k_stop * (float)T), inv_L));
     {
         int first = 4;           // (every wavefront reduces the S <= 128 stream lengths on its own)
