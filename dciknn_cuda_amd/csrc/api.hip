@@ -91,7 +91,7 @@ struct dcih_index {
     uint16_t* d_lids = nullptr;         // [I][n] partition-relative ids (partitions <= 65536 points)
     float* d_own = nullptr;             // rows copied in by dcih_append (the index owns these)
     int64_t own_rows = 0;               // capacity of d_own in rows
-    float* d_stop_hint = nullptr;       // [2][block_size] epoch-size hints learnt from earlier queries
+    float* d_stop_hint = nullptr;       // [3][block_size] epoch-size hints learnt from earlier queries
     int hint_k = 0, hint_outer = 0, hint_T = 0, hint_maxc = 0;   // query shape the hints belong to
     int traversal = 0;                  // DCIH_OPT_TRAVERSAL value
     unsigned long long* d_phase_ticks = nullptr;   // optional profile of the batch kernel
@@ -249,7 +249,7 @@ static int build_index(dcih_index* h, int64_t num_points, const float* d_data, i
     const size_t b_ids = align_up(cells * sizeof(int32_t));
     // +16: the traversal reads whole aligned 16-byte chunks, also at the very end
     const size_t b_lids = small_parts ? align_up((cells + 16) * sizeof(uint16_t)) : 0;
-    const size_t b_hint = align_up((size_t)2 * block_size * sizeof(float));   // stop step, promotions at the stop
+    const size_t b_hint = align_up((size_t)3 * block_size * sizeof(float));   // stop step, promotions at the stop, stops seen
     int rc = ensure_arena(h, 3 * b_keys + b_lids + b_hint);
     if (rc) return rc;
     rc = ensure_ws(h, b_keys + align_up(tmp_bytes));
@@ -263,7 +263,7 @@ static int build_index(dcih_index* h, int64_t num_points, const float* d_data, i
     float* d_keys = (float*)h->ws;
     void* d_tmp = tmp_bytes ? (void*)((char*)h->ws + b_keys) : nullptr;
     do {
-        if (hipMemsetAsync(h->d_stop_hint, 0, (size_t)2 * block_size * sizeof(float), s) != hipSuccess) {
+        if (hipMemsetAsync(h->d_stop_hint, 0, (size_t)3 * block_size * sizeof(float), s) != hipSuccess) {
             rc = fail(DCIH_EHIP, "build: clearing the hint table failed");
             break;
         }
@@ -372,7 +372,7 @@ int dcih_query(dcih_index* h, int dim, int num_queries, const float* d_query,
     // the hints describe where traversals of one query shape stop; forget them when it changes
     if (h->hint_k != num_neighbours || h->hint_outer != num_outer_iterations ||
         h->hint_T != thread_size || h->hint_maxc != max_num_candidates) {
-        DCIH_HIP(hipMemsetAsync(h->d_stop_hint, 0, (size_t)2 * block_size * sizeof(float), s));
+        DCIH_HIP(hipMemsetAsync(h->d_stop_hint, 0, (size_t)3 * block_size * sizeof(float), s));
         h->hint_k = num_neighbours; h->hint_outer = num_outer_iterations;
         h->hint_T = thread_size; h->hint_maxc = max_num_candidates;
     }

@@ -47,7 +47,7 @@ struct QueryArgs {
     uint32_t* redo_count;    // their number
     const int32_t* item_list;    // step-by-step kernel: null = all nq*B items, else this list
     const uint32_t* item_count;  // ... of this length
-    float* stop_hint;        // null, or [2][B] running averages per partition: stop step, promotions at the stop
+    float* stop_hint;        // null, or [3][B] per partition: running averages of the stop step and of the promotions at the stop, stops seen
     unsigned long long* phase_ticks;  // null, or 16 accumulators for the batch kernel's phases
     int mode;                // 0 = pick, 1 = step-by-step kernel, 2 = batch kernel
     int32_t* out_ids;        // [nq][k]

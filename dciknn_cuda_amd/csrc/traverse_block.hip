@@ -1005,11 +1005,14 @@ __global__ __launch_bounds__(NT, MINW) void traverse_block_kernel(QueryArgs a, B
     }
     if (a.stop_hint && tid == 0 && misc[kStop]) {
         const float cur = (float)((((unsigned long long)misc[kStopStepHi] << 32) | misc[kStopStepLo]) + 1);
-        const float old = a.stop_hint[b];     // racy on purpose: any recent value will do
-        a.stop_hint[b] = old > 0.0f ? 0.75f * old + 0.25f * cur : cur;
+        // racy on purpose: any recent value will do.  The mean of the first 50 stops, then an
+        // exponential average with weight 1/50 (a smooth hint wastes the fewest epochs).
+        const float seen_stops = a.stop_hint[2 * a.B + b];
+        const float w = 1.0f / fminf(seen_stops + 1.0f, 50.0f);
+        a.stop_hint[2 * a.B + b] = fminf(seen_stops + 1.0f, 1.0e6f);
+        a.stop_hint[b] += w * (cur - a.stop_hint[b]);
         const float curp = (float)(misc[kNumCand] + misc[kEventCount]);
-        const float oldp = a.stop_hint[a.B + b];
-        a.stop_hint[a.B + b] = oldp > 0.0f ? 0.75f * oldp + 0.25f * curp : curp;
+        a.stop_hint[a.B + b] += w * (curp - a.stop_hint[a.B + b]);
     }
     // ---- results -------------------------------------------------------------------
     const int topn = (int)misc[kTopN];
