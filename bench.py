@@ -32,7 +32,7 @@ HBM_PEAK_GBS = 8000.0   # MI355X HBM3E
 # (2.000 and 1.000); the counter runs are summarised in profiles/bench_c2_hbm_traffic.txt.
 # Counters cannot be read from inside this process, so the figure is a constant
 # tied to that exact configuration and omitted for any other.
-MEASURED_TRAFFIC_C2_DEFAULT = 59.7e9
+MEASURED_TRAFFIC_C2_DEFAULT = 49.3e9
 
 # (block_size, thread_size, num_outer_iterations) used when none are given:
 # the fastest setting found with recall@k >= 0.95 on that workload.

@@ -87,7 +87,7 @@ struct dcih_index {
     int block_size = 0;
     float* d_skeys = nullptr;           // [I][n]
     int32_t* d_sids = nullptr;          // [I][n]
-    uint32_t* d_inv = nullptr;          // [I][n] position of each point in its sorted slice
+    uint16_t* d_inv = nullptr;          // [I][n] position of each point in its sorted slice (partitions <= 65536 points)
     uint16_t* d_lids = nullptr;         // [I][n] partition-relative ids (partitions <= 65536 points)
     float* d_own = nullptr;             // rows copied in by dcih_append (the index owns these)
     int64_t own_rows = 0;               // capacity of d_own in rows
@@ -250,16 +250,17 @@ static int build_index(dcih_index* h, int64_t num_points, const float* d_data, i
     // +16: the traversal reads whole aligned 16-byte chunks, also at the very end
     const size_t b_lids = small_parts ? align_up((cells + 16) * sizeof(uint16_t)) : 0;
     const size_t b_hint = align_up((size_t)3 * block_size * sizeof(float));   // stop step, promotions at the stop, stops seen
-    int rc = ensure_arena(h, 3 * b_keys + b_lids + b_hint);
+    const size_t b_inv = small_parts ? align_up(cells * sizeof(uint16_t)) : 0;
+    int rc = ensure_arena(h, b_keys + b_ids + b_inv + b_lids + b_hint);
     if (rc) return rc;
     rc = ensure_ws(h, b_keys + align_up(tmp_bytes));
     if (rc) return rc;
     char* base = (char*)h->arena;
     h->d_skeys = (float*)base;
     h->d_sids = (int32_t*)(base + b_keys);
-    h->d_inv = (uint32_t*)(base + b_keys + b_ids);
-    h->d_lids = small_parts ? (uint16_t*)(base + 3 * b_keys) : nullptr;
-    h->d_stop_hint = (float*)(base + 3 * b_keys + b_lids);
+    h->d_inv = small_parts ? (uint16_t*)(base + b_keys + b_ids) : nullptr;
+    h->d_lids = small_parts ? (uint16_t*)(base + b_keys + b_ids + b_inv) : nullptr;
+    h->d_stop_hint = (float*)(base + b_keys + b_ids + b_inv + b_lids);
     float* d_keys = (float*)h->ws;
     void* d_tmp = tmp_bytes ? (void*)((char*)h->ws + b_keys) : nullptr;
     do {

@@ -40,7 +40,7 @@ __device__ inline unsigned long long pack_key(float key, uint32_t pos) {
 template <bool FINAL>
 __global__ void segsort_tile_kernel(const float* __restrict__ keys, SegGeom g,
                                     float* __restrict__ skeys, int32_t* __restrict__ sids,
-                                    uint32_t* __restrict__ inv, uint16_t* __restrict__ lids,
+                                    uint16_t* __restrict__ inv, uint16_t* __restrict__ lids,
                                     unsigned long long* __restrict__ packed, int np2) {
     extern __shared__ unsigned long long s[];
     const int64_t flat = blockIdx.x;
@@ -86,7 +86,7 @@ __global__ void segsort_tile_kernel(const float* __restrict__ keys, SegGeom g,
             if (j < m) pos_of[local[r]] = (uint32_t)j;
         }
         __syncthreads();
-        for (int j = threadIdx.x; j < m; j += blockDim.x) inv[base + j] = pos_of[j];
+        for (int j = threadIdx.x; j < m; j += blockDim.x) inv[base + j] = (uint16_t)pos_of[j];
     }
 }
 
@@ -114,7 +114,7 @@ template <int kRadixThreads, int IPT>
 // (256 threads with more than 45 items each: registers for two workgroups per CU)
 __global__ __launch_bounds__(kRadixThreads, (kRadixThreads == 256 && IPT > 45) ? 2 : 1) void segsort_radix_kernel(
     const float* __restrict__ keys, SegGeom g, float* __restrict__ skeys,
-    int32_t* __restrict__ sids, uint32_t* __restrict__ inv, uint16_t* __restrict__ lids,
+    int32_t* __restrict__ sids, uint16_t* __restrict__ inv, uint16_t* __restrict__ lids,
     unsigned long long* __restrict__ packed) {
     extern __shared__ uint32_t rs[];
     uint32_t* stage = rs;                                         // IPT*1024 words
@@ -300,7 +300,7 @@ __global__ __launch_bounds__(kRadixThreads, (kRadixThreads == 256 && IPT > 45) ?
 
 template <int NT, int IPT>
 static int launch_radix(const float* d_keys, const SegGeom& g, int num_indices, float* d_skeys,
-                        int32_t* d_sids, uint32_t* d_inv, uint16_t* d_lids,
+                        int32_t* d_sids, uint16_t* d_inv, uint16_t* d_lids,
                         unsigned long long* d_packed, hipStream_t s) {
     const size_t lds = (size_t)(IPT * NT + 8 * NT + 64) * sizeof(uint32_t);
     static DeviceOnce once;
@@ -351,7 +351,7 @@ __device__ inline int64_t merge_split_wave(const unsigned long long* __restrict_
 __global__ __launch_bounds__(kMergeThreads) void segsort_merge_kernel(
     const unsigned long long* __restrict__ src, unsigned long long* __restrict__ dst,
     SegGeom g, int chunks, int64_t run, float* __restrict__ skeys, int32_t* __restrict__ sids,
-    uint32_t* __restrict__ inv, uint16_t* __restrict__ lids) {
+    uint16_t* __restrict__ inv, uint16_t* __restrict__ lids) {
     __shared__ unsigned long long s_in[kMergeChunk];
     __shared__ unsigned long long s_out[kMergeChunk];
     __shared__ int64_t s_split[2];
@@ -417,7 +417,7 @@ __global__ __launch_bounds__(kMergeThreads) void segsort_merge_kernel(
             const int64_t e = out0 + j;
             skeys[e] = ord2f((uint32_t)(w >> 32));
             sids[e] = (int32_t)(off + (uint32_t)w);
-            if (inv) inv[base + (uint32_t)w] = (uint32_t)(ps + d0 + j);
+            if (inv) inv[base + (uint32_t)w] = (uint16_t)(ps + d0 + j);
             if (lids) lids[e] = (uint16_t)(uint32_t)w;
         }
     }
@@ -436,7 +436,7 @@ static int next_pow2(int v) {
 }
 
 int segsort(const float* d_keys, int num_indices, int64_t n, int block_size,
-            float* d_skeys, int32_t* d_sids, uint32_t* d_inv, uint16_t* d_lids, void* d_tmp,
+            float* d_skeys, int32_t* d_sids, uint16_t* d_inv, uint16_t* d_lids, void* d_tmp,
             hipStream_t s) {
     if (n <= 0) return 0;
     SegGeom g;
