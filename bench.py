@@ -92,6 +92,8 @@ def run_c5(a):
     other, the fixed query batch run after each; one JSON line with per-size figures."""
     import numpy as np
     import torch
+    from dciknn_cuda_amd import build as engine_build
+    engine_build.ensure_built()      # loads what is built; compiles only in a tree without libraries
     import dciknn_cuda_amd as D
     from dciknn_cuda_amd import workloads
     cfg = dict(TUNED["c5"])
@@ -151,6 +153,8 @@ def main():
     if not torch.cuda.is_available():
         print("bench.py needs a GPU", file=sys.stderr)
         sys.exit(1)
+    from dciknn_cuda_amd import build as engine_build
+    engine_build.ensure_built()      # loads what is built; compiles only in a tree without libraries
     import dciknn_cuda_amd as D
     from dciknn_cuda_amd import _capi, workloads
 

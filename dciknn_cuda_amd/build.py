@@ -82,5 +82,13 @@ def build_all(verbose=False):
     return build_library(verbose), build_extension(verbose)
 
 
+def ensure_built():
+    """Build the two libraries if either is missing (tests, smoke and benchmark call
+    this; they never rebuild what is there)."""
+    if not (os.path.exists(LIB) and os.path.exists(EXT)):
+        build_all()
+    return LIB, EXT
+
+
 if __name__ == "__main__":
     print(build_all(verbose=True))

@@ -10,6 +10,9 @@ if ROOT not in sys.path:
 
 def pytest_configure(config):
     config.addinivalue_line("markers", "gpu: needs a real MI355X (run with -m gpu)")
+    # the tests load what is built; only a tree without libraries compiles them first
+    from dciknn_cuda_amd import build
+    build.ensure_built()
 
 
 @pytest.fixture(scope="session")
