@@ -409,7 +409,14 @@ int dcih_query(dcih_index* h, int dim, int num_queries, const float* d_query,
         mark(h, DCIH_T_TRAVERSE, 1, s);
         return rc;
     }
-    if (!blind && num_neighbours > 8192) {
+    // The stop rule (:598-607) can also never fire when a partition has fewer points than
+    // max_num_candidates and fewer windows per simple index (at most ppb / T + 3) than
+    // num_outer_iterations: the loop then runs every partition dry, as in the reference's own
+    // example (3000 points in 100 partitions, 5000 iterations).  Left to pick, the engine
+    // computes that answer directly as well.
+    const bool runs_dry = !blind && h->traversal == 0 && a.ppb < (int64_t)max_num_candidates &&
+                          a.ppb / thread_size + 4 < (int64_t)num_outer_iterations;
+    if (!blind && (num_neighbours > 8192 || runs_dry)) {
         // With more neighbours asked for than a partition holds, no partition can stop early
         // (c0 counts promotions of one partition, :598-607), so the answer is the full ranking
         // and is computed as such.  (With exactly as many, the results are the same but the

@@ -132,7 +132,10 @@ int dcih_append(dcih_index* h, int dim, int64_t num_points, const float* d_data,
  * promoted, and the result, the num_neighbours closest of all points by (distance,
  * id), is computed directly (all distances, summed in index order like
  * compute_dist_device, :36-44; one sort per query; the counters from their closed
- * forms).  Above 8192 otherwise, the traversal records every candidate's distance
+ * forms).  The same direct computation is used for any num_neighbours when the stop
+ * rule provably cannot fire (a partition holds fewer points than max_num_candidates
+ * and fewer windows per simple index than num_outer_iterations) and the kernel
+ * choice is left automatic.  Above 8192 otherwise, the traversal records every candidate's distance
  * in a row of num_points cells per query and the rows are sorted; both paths work
  * through the queries in chunks and use up to 2 GB of workspace.
  *
