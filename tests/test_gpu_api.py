@@ -262,3 +262,40 @@ def test_large_k_with_early_stops(gpu, oracle, n, B, T, k, outer):
     np.testing.assert_allclose(dists, ref["dists"], rtol=1e-5)
     if B == 2 and T == 1:
         assert np.all(ctr[:, 1] < n), "the case is meant to stop before everything is promoted"
+
+
+def test_query_can_be_captured_in_a_graph(gpu):
+    """After one warm-up call (workspace sized, hints of this query shape in place) a
+    dcih_query enqueues only kernels, so a HIP graph can hold it: every replay, with
+    eager calls in between, gives the eager result."""
+    from dciknn_cuda_amd import _capi
+    X, Q = _xy(n=30000, nq=32, dim=16, seed=5)
+    dci = gpu.DCI(16, 2, 5, 8, 4, seed=9)
+    dci.add(X)
+    nq, k = Q.shape[0], 7
+    ids = torch.empty((nq, k), dtype=torch.int32, device="cuda")
+    dists = torch.empty((nq, k), dtype=torch.float32, device="cuda")
+
+    def call(stream):
+        _capi.check(dci._lib.dcih_query(dci._dci_inst, 16, nq, Q.data_ptr(), k, 0, 60, 10 * k, 8, 4,
+                                        ids.data_ptr(), dists.data_ptr(), None, stream))
+    s = torch.cuda.Stream()
+    with torch.cuda.stream(s):
+        call(s.cuda_stream)
+        call(s.cuda_stream)
+    s.synchronize()
+    want_ids, want_dists = ids.clone(), dists.clone()
+    g = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(g, stream=s):
+        call(torch.cuda.current_stream().cuda_stream)
+    for _ in range(4):
+        ids.fill_(-5)
+        dists.fill_(-5.0)
+        torch.cuda.synchronize()
+        g.replay()
+        torch.cuda.synchronize()
+        assert torch.equal(ids, want_ids) and torch.equal(dists, want_dists)
+        call(0)                                # eager work between the replays
+        torch.cuda.synchronize()
+    del g
+    dci.free()
