@@ -32,6 +32,9 @@ SIGNATURES = {
     "dcih_query": (_c.c_int, [_c.c_void_p, _c.c_int, _c.c_int, _c.c_void_p, _c.c_int,
                               _c.c_int, _c.c_int, _c.c_int, _c.c_int, _c.c_int,
                               _c.c_void_p, _c.c_void_p, _c.c_void_p, _c.c_void_p]),
+    "dcih_debug_launch_map": (_c.c_int64, [_c.c_int, _c.c_int, _c.c_int, _c.c_int64,
+                                           _c.POINTER(_c.c_int), _c.POINTER(_c.c_int),
+                                           _c.POINTER(_c.c_int)]),
     "dcih_get_index": (_c.c_int, [_c.c_void_p, _c.c_void_p, _c.c_void_p]),
     "dcih_set_option": (_c.c_int, [_c.c_void_p, _c.c_int, _c.c_int]),
     "dcih_phase_profile": (_c.c_int, [_c.c_void_p, _c.c_void_p]),

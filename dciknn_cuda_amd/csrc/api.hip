@@ -5,6 +5,7 @@
 // returns status codes instead of asserting, takes a stream, frees what it
 // allocates, and launches a constant number of kernels per call instead of
 // several per query.
+#include <algorithm>
 #include <cmath>
 #include <cstring>
 #include <new>
@@ -78,6 +79,7 @@ using namespace dcih;
 
 struct dcih_index {
     int dim = 0, M = 0, L = 0, device = 0;
+    int xcds = 8;                       // accelerator dies of the device
     uint64_t seed = 0;
     uint64_t draws = 0;                 // direction sets drawn so far
     std::vector<float> h_dirs;          // [I][dim]
@@ -90,7 +92,9 @@ struct dcih_index {
     uint16_t* d_inv = nullptr;          // [I][n] position of each point in its sorted slice (partitions <= 65536 points)
     uint16_t* d_lids = nullptr;         // [I][n] partition-relative ids (partitions <= 65536 points)
     float* d_own = nullptr;             // rows copied in by dcih_append (the index owns these)
-    int64_t own_rows = 0;               // capacity of d_own in rows
+    float* d_ukeys = nullptr;           // [I][own_rows] unsorted projections of the rows in d_own
+    int64_t own_rows = 0;               // capacity of d_own / d_ukeys in rows
+    int64_t ukeys_rows = 0;             // leading rows of d_own whose projections d_ukeys holds
     float* d_stop_hint = nullptr;       // [3][block_size] epoch-size hints learnt from earlier queries
     int hint_k = 0, hint_outer = 0, hint_T = 0, hint_maxc = 0;   // query shape the hints belong to
     int traversal = 0;                  // DCIH_OPT_TRAVERSAL value
@@ -98,10 +102,13 @@ struct dcih_index {
     // grow-only workspace: query scratch, and the unsorted keys during a build
     void* ws = nullptr;
     size_t ws_bytes = 0;
-    // grow-only arena the sorted arrays and the hint table are carved from; kept
-    // across dcih_clear so that a rebuild allocates nothing
-    void* arena = nullptr;
-    size_t arena_bytes = 0;
+    // grow-only arenas the sorted arrays and the hint table are carved from; kept
+    // across dcih_clear so that a rebuild allocates nothing.  The index lives in
+    // arena[cur]; dcih_append builds the next one in the other and then switches, so
+    // a failed append leaves the index as it was.
+    void* arena[2] = {nullptr, nullptr};
+    size_t arena_bytes[2] = {0, 0};
+    int cur = 0;
     // optional per-kernel timing: ev[2*t], ev[2*t+1] bracket timer t
     bool profiling = false;
     hipEvent_t ev[2 * DCIH_NUM_TIMERS] = {};
@@ -145,21 +152,33 @@ int release_sorted(dcih_index* h) {
 
 int release_arena(dcih_index* h) {
     (void)release_sorted(h);
-    if (h->arena) { DCIH_HIP(hipFree(h->arena)); h->arena = nullptr; h->arena_bytes = 0; }
+    for (int j = 0; j < 2; j++)
+        if (h->arena[j]) { (void)hipFree(h->arena[j]); h->arena[j] = nullptr; h->arena_bytes[j] = 0; }
     return 0;
 }
 
 int release_index(dcih_index* h) {
     const int rc = release_sorted(h);
-    if (h->d_own) { (void)hipFree(h->d_own); h->d_own = nullptr; h->own_rows = 0; }
+    if (h->d_own) { (void)hipFree(h->d_own); h->d_own = nullptr; }
+    if (h->d_ukeys) { (void)hipFree(h->d_ukeys); h->d_ukeys = nullptr; }
+    h->own_rows = h->ukeys_rows = 0;
     h->d_data = nullptr;
     h->n = 0;
     h->block_size = 0;
     return rc;
 }
 
-int ensure_ws(dcih_index* h, size_t bytes) {
+// True while `s` is recording into a graph: nothing may be allocated or freed then.
+bool capturing(hipStream_t s) {
+    hipStreamCaptureStatus st = hipStreamCaptureStatusNone;
+    return hipStreamIsCapturing(s, &st) == hipSuccess && st != hipStreamCaptureStatusNone;
+}
+
+int ensure_ws(dcih_index* h, size_t bytes, hipStream_t s) {
     if (bytes <= h->ws_bytes) return 0;
+    if (capturing(s))
+        return fail(DCIH_ESTATE, "the workspace would have to grow while the stream is being captured: "
+                                 "run the same call once outside the capture first");
     if (h->ws) { DCIH_HIP(hipFree(h->ws)); h->ws = nullptr; h->ws_bytes = 0; }
     DCIH_HIP(hipMalloc(&h->ws, bytes));
     h->ws_bytes = bytes;
@@ -168,12 +187,38 @@ int ensure_ws(dcih_index* h, size_t bytes) {
 
 size_t align_up(size_t v) { return (v + 255) & ~(size_t)255; }
 
-int ensure_arena(dcih_index* h, size_t bytes) {
-    if (bytes <= h->arena_bytes) return 0;
-    if (h->arena) { DCIH_HIP(hipFree(h->arena)); h->arena = nullptr; h->arena_bytes = 0; }
-    DCIH_HIP(hipMalloc(&h->arena, bytes));
-    h->arena_bytes = bytes;
+// Makes arena `which` at least `bytes` large.  Growing frees that arena first, so it must
+// not hold the live index.
+int ensure_arena(dcih_index* h, int which, size_t bytes) {
+    if (bytes <= h->arena_bytes[which]) return 0;
+    if (h->arena[which]) { DCIH_HIP(hipFree(h->arena[which])); h->arena[which] = nullptr; h->arena_bytes[which] = 0; }
+    DCIH_HIP(hipMalloc(&h->arena[which], bytes));
+    h->arena_bytes[which] = bytes;
     return 0;
+}
+
+// Where the arrays of an index of n points lie inside an arena.
+struct ArenaLayout {
+    size_t keys, ids, inv, lids, hint, total;   // byte offsets, and the size of it all
+    bool small_parts;                           // partitions of at most 65536 points: 16-bit tables exist
+};
+ArenaLayout arena_layout(int I, int64_t n, int block_size) {
+    ArenaLayout y;
+    const size_t cells = (size_t)I * (size_t)n;
+    y.small_parts = (n + block_size - 1) / block_size <= 65536;
+    const size_t b_keys = align_up(cells * sizeof(float));
+    const size_t b_ids = align_up(cells * sizeof(int32_t));
+    const size_t b_inv = y.small_parts ? align_up(cells * sizeof(uint16_t)) : 0;
+    // +16: the traversal reads whole aligned 16-byte chunks, also at the very end
+    const size_t b_lids = y.small_parts ? align_up((cells + 16) * sizeof(uint16_t)) : 0;
+    const size_t b_hint = align_up((size_t)3 * block_size * sizeof(float));   // stop step, promotions at the stop, stops seen
+    y.keys = 0;
+    y.ids = b_keys;
+    y.inv = y.ids + b_ids;
+    y.lids = y.inv + b_inv;
+    y.hint = y.lids + b_lids;
+    y.total = y.hint + b_hint;
+    return y;
 }
 
 // Records the start (which = 0) or end (1) event of timer t when profiling.
@@ -208,6 +253,12 @@ int dcih_create(int dim, int num_comp_indices, int num_simp_indices, int device,
     if (!h) return fail(DCIH_EHIP, "dcih_create: out of host memory");
     h->dim = dim; h->M = num_comp_indices; h->L = num_simp_indices;
     h->device = device; h->seed = seed;
+    {   // dies with an L2 of their own: the batch traversal orders its work by them
+        int xcds = 0;
+        if (hipDeviceGetAttribute(&xcds, hipDeviceAttributeNumberOfXccs, device) == hipSuccess && xcds >= 1)
+            h->xcds = xcds;
+        (void)hipGetLastError();
+    }
     const size_t bytes = (size_t)num_indices(h) * dim * sizeof(float);
     if (hipMalloc(&h->d_dirs, bytes) != hipSuccess) {
         delete h;
@@ -234,53 +285,35 @@ int dcih_set_directions(dcih_index* h, const float* h_dirs) {
     return DCIH_OK;
 }
 
-// Projects and sorts `num_points` rows at d_data into a fresh index (the handle holds
-// no sorted arrays when this is called).  Synchronises the stream before returning.
-static int build_index(dcih_index* h, int64_t num_points, const float* d_data, int block_size,
-                       hipStream_t s) {
+// Sorts the projections of `num_points` rows (index i's at d_keys + i * key_stride) into
+// arena `which`, which must already be large enough, and makes the result the handle's
+// index over the rows at d_data.  Synchronises the stream before returning; on failure the
+// handle's fields are untouched.
+static int sort_into(dcih_index* h, int which, const float* d_keys, int64_t key_stride,
+                     int64_t num_points, const float* d_data, int block_size, void* d_tmp,
+                     hipStream_t s) {
     const int I = num_indices(h);
-    const int dim = h->dim;
-    const size_t cells = (size_t)I * num_points;
-    const size_t tmp_bytes = segsort_tmp_bytes(I, num_points, block_size);
-    const bool small_parts = (num_points + block_size - 1) / block_size <= 65536;
-    // one arena for what the index keeps, the workspace for what only the build needs:
-    // a rebuild of the same size allocates and frees nothing
-    const size_t b_keys = align_up(cells * sizeof(float));
-    const size_t b_ids = align_up(cells * sizeof(int32_t));
-    // +16: the traversal reads whole aligned 16-byte chunks, also at the very end
-    const size_t b_lids = small_parts ? align_up((cells + 16) * sizeof(uint16_t)) : 0;
-    const size_t b_hint = align_up((size_t)3 * block_size * sizeof(float));   // stop step, promotions at the stop, stops seen
-    const size_t b_inv = small_parts ? align_up(cells * sizeof(uint16_t)) : 0;
-    int rc = ensure_arena(h, b_keys + b_ids + b_inv + b_lids + b_hint);
-    if (rc) return rc;
-    rc = ensure_ws(h, b_keys + align_up(tmp_bytes));
-    if (rc) return rc;
-    char* base = (char*)h->arena;
-    h->d_skeys = (float*)base;
-    h->d_sids = (int32_t*)(base + b_keys);
-    h->d_inv = small_parts ? (uint16_t*)(base + b_keys + b_ids) : nullptr;
-    h->d_lids = small_parts ? (uint16_t*)(base + b_keys + b_ids + b_inv) : nullptr;
-    h->d_stop_hint = (float*)(base + b_keys + b_ids + b_inv + b_lids);
-    float* d_keys = (float*)h->ws;
-    void* d_tmp = tmp_bytes ? (void*)((char*)h->ws + b_keys) : nullptr;
-    do {
-        if (hipMemsetAsync(h->d_stop_hint, 0, (size_t)3 * block_size * sizeof(float), s) != hipSuccess) {
-            rc = fail(DCIH_EHIP, "build: clearing the hint table failed");
-            break;
-        }
-        mark(h, DCIH_T_PROJECT, 0, s);
-        rc = project(h->d_dirs, I, d_data, num_points, dim, d_keys, s);
-        mark(h, DCIH_T_PROJECT, 1, s);
-        if (rc) break;
+    const ArenaLayout y = arena_layout(I, num_points, block_size);
+    char* base = (char*)h->arena[which];
+    float* skeys = (float*)(base + y.keys);
+    int32_t* sids = (int32_t*)(base + y.ids);
+    uint16_t* inv = y.small_parts ? (uint16_t*)(base + y.inv) : nullptr;
+    uint16_t* lids = y.small_parts ? (uint16_t*)(base + y.lids) : nullptr;
+    float* hint = (float*)(base + y.hint);
+    // (the table's room is a multiple of 256 bytes, so whole 64-bit words may be cleared)
+    int rc = zero_words64(hint, (int64_t)(((size_t)3 * block_size * sizeof(float) + 7) / 8), s);
+    if (rc == DCIH_OK) {
         mark(h, DCIH_T_SEGSORT, 0, s);
-        rc = segsort(d_keys, I, num_points, block_size, h->d_skeys, h->d_sids, h->d_inv, h->d_lids, d_tmp, s);
+        rc = segsort(d_keys, key_stride, I, num_points, block_size, skeys, sids, inv, lids, d_tmp, s);
         mark(h, DCIH_T_SEGSORT, 1, s);
-    } while (0);
+    }
     // like the reference's dci_add, the call returns when the index is complete
     const hipError_t se = hipStreamSynchronize(s);
     if (rc == DCIH_OK && se != hipSuccess)
         rc = fail(DCIH_EHIP, std::string("build: ") + hipGetErrorString(se));
     if (rc) return rc;
+    h->d_skeys = skeys; h->d_sids = sids; h->d_inv = inv; h->d_lids = lids; h->d_stop_hint = hint;
+    h->cur = which;
     h->d_data = d_data;
     h->n = num_points;
     h->block_size = block_size;
@@ -298,7 +331,25 @@ int dcih_add(dcih_index* h, int dim, int64_t num_points, const float* d_data,
     if (block_size <= 0 || thread_size <= 0)
         return fail(DCIH_EINVAL, "dcih_add: block_size and thread_size must be positive");
     DeviceGuard guard(h->device);
-    const int rc = build_index(h, num_points, d_data, block_size, (hipStream_t)stream);
+    hipStream_t s = (hipStream_t)stream;
+    const int I = num_indices(h);
+    // one arena for what the index keeps, the workspace for what only the build needs
+    // (the unsorted keys): a rebuild of the same size allocates and frees nothing
+    const size_t b_keys = align_up((size_t)I * num_points * sizeof(float));
+    const size_t tmp_bytes = segsort_tmp_bytes(I, num_points, block_size);
+    int rc = ensure_arena(h, h->cur, arena_layout(I, num_points, block_size).total);
+    if (rc == DCIH_OK) rc = ensure_ws(h, b_keys + align_up(tmp_bytes), s);
+    if (rc == DCIH_OK) {
+        float* d_keys = (float*)h->ws;
+        mark(h, DCIH_T_PROJECT, 0, s);
+        rc = project(h->d_dirs, I, d_data, num_points, dim, d_keys, num_points, s);
+        mark(h, DCIH_T_PROJECT, 1, s);
+        if (rc == DCIH_OK)
+            rc = sort_into(h, h->cur, d_keys, num_points, num_points, d_data, block_size,
+                           tmp_bytes ? (void*)((char*)h->ws + b_keys) : nullptr, s);
+        else
+            (void)hipStreamSynchronize(s);
+    }
     if (rc) (void)release_index(h);
     return rc;
 }
@@ -316,64 +367,125 @@ int dcih_append(dcih_index* h, int dim, int64_t num_points, const float* d_data,
     if (total > 0x7fffffffLL) return fail(DCIH_EINVAL, "dcih_append: more than 2^31-1 points");
     DeviceGuard guard(h->device);
     hipStream_t s = (hipStream_t)stream;
+    const int I = num_indices(h);
     const size_t row_bytes = (size_t)dim * sizeof(float);
-    // all rows move into one buffer the index owns (capacity doubles, so copies amortise)
-    if (!h->d_own || h->own_rows < total) {
-        const int64_t cap = std::max<int64_t>(total, 2 * h->own_rows);
-        float* fresh = nullptr;
-        DCIH_HIP(hipMalloc(&fresh, (size_t)cap * row_bytes));
-        if (h->n > 0)
-            DCIH_HIP(hipMemcpyAsync(fresh, h->d_data, (size_t)h->n * row_bytes, hipMemcpyDeviceToDevice, s));
-        DCIH_HIP(hipStreamSynchronize(s));
-        if (h->d_own) (void)hipFree(h->d_own);
-        h->d_own = fresh;
-        h->own_rows = cap;
-    } else if (h->n > 0 && h->d_data != h->d_own) {
-        DCIH_HIP(hipMemcpyAsync(h->d_own, h->d_data, (size_t)h->n * row_bytes, hipMemcpyDeviceToDevice, s));
+
+    // Everything that can fail for lack of memory happens before the index is touched:
+    // room for the rows and their projections (both owned by the index, capacity doubles
+    // so that copies amortise), for the next index in the spare arena, and for the sort.
+    float* rows = h->d_own;
+    float* ukeys = h->d_ukeys;
+    int64_t cap = h->own_rows;
+    int64_t have_keys = (h->n > 0 && h->d_data == h->d_own) ? std::min(h->ukeys_rows, h->n) : 0;
+    float* fresh_rows = nullptr;
+    float* fresh_keys = nullptr;
+    if (!rows || cap < total) {
+        cap = std::max<int64_t>(total, 2 * h->own_rows);
+        if (hipMalloc(&fresh_rows, (size_t)cap * row_bytes) != hipSuccess ||
+            hipMalloc(&fresh_keys, (size_t)I * cap * sizeof(float)) != hipSuccess) {
+            (void)hipGetLastError();
+            if (fresh_rows) (void)hipFree(fresh_rows);
+            return fail(DCIH_EHIP, "dcih_append: out of device memory for the rows (the index is unchanged)");
+        }
+        rows = fresh_rows;
+        ukeys = fresh_keys;
     }
-    DCIH_HIP(hipMemcpyAsync(h->d_own + (size_t)h->n * dim, d_data, (size_t)num_points * row_bytes,
-                            hipMemcpyDeviceToDevice, s));
-    // the partition boundaries move with the total, so every slice is rebuilt
-    DCIH_HIP(hipStreamSynchronize(s));
-    int rc = release_sorted(h);
-    if (rc) return rc;
-    rc = build_index(h, total, h->d_own, block_size, s);
-    if (rc) (void)release_index(h);
-    return rc;
+    const int spare = 1 - h->cur;
+    const size_t tmp_bytes = segsort_tmp_bytes(I, total, block_size);
+    int rc = ensure_arena(h, h->n > 0 ? spare : h->cur,
+                          std::max(arena_layout(I, total, block_size).total,
+                                   arena_layout(I, cap, block_size).total));
+    if (rc == DCIH_OK && tmp_bytes) rc = ensure_ws(h, align_up(tmp_bytes), s);
+    hipError_t e = hipSuccess;
+    if (rc == DCIH_OK && h->n > 0 && rows != h->d_data)        // rows (and projections) indexed so far
+        e = hipMemcpyAsync(rows, h->d_data, (size_t)h->n * row_bytes, hipMemcpyDeviceToDevice, s);
+    if (rc == DCIH_OK && e == hipSuccess && have_keys > 0 && ukeys != h->d_ukeys)
+        e = hipMemcpy2DAsync(ukeys, (size_t)cap * sizeof(float), h->d_ukeys, (size_t)h->own_rows * sizeof(float),
+                             (size_t)have_keys * sizeof(float), (size_t)I, hipMemcpyDeviceToDevice, s);
+    if (rc == DCIH_OK && e == hipSuccess)
+        e = hipMemcpyAsync(rows + (size_t)h->n * dim, d_data, (size_t)num_points * row_bytes,
+                           hipMemcpyDeviceToDevice, s);
+    if (rc == DCIH_OK && e != hipSuccess) rc = fail(DCIH_EHIP, std::string("dcih_append: ") + hipGetErrorString(e));
+    if (rc == DCIH_OK) {
+        // only rows without kept projections are projected: the new ones, after a plain
+        // dcih_add (which keeps none) all of them
+        mark(h, DCIH_T_PROJECT, 0, s);
+        rc = project(h->d_dirs, I, rows + (size_t)have_keys * dim, total - have_keys, dim,
+                     ukeys + have_keys, cap, s);
+        mark(h, DCIH_T_PROJECT, 1, s);
+    }
+    if (rc == DCIH_OK)
+        // the partition boundaries move with the total, so every slice is formed again
+        rc = sort_into(h, h->n > 0 ? spare : h->cur, ukeys, cap, total, rows, block_size,
+                       tmp_bytes ? h->ws : nullptr, s);
+    else
+        (void)hipStreamSynchronize(s);
+    if (rc) {       // the index stays as it was
+        if (fresh_rows) (void)hipFree(fresh_rows);
+        if (fresh_keys) (void)hipFree(fresh_keys);
+        return rc;
+    }
+    if (fresh_rows) {
+        if (h->d_own) (void)hipFree(h->d_own);
+        if (h->d_ukeys) (void)hipFree(h->d_ukeys);
+        h->d_own = fresh_rows;
+        h->d_ukeys = fresh_keys;
+        h->own_rows = cap;
+    }
+    h->ukeys_rows = total;
+    return DCIH_OK;
 }
 
-int dcih_query(dcih_index* h, int dim, int num_queries, const float* d_query,
-               int num_neighbours, int blind, int num_outer_iterations,
-               int max_num_candidates, int block_size, int thread_size,
-               int32_t* d_nn, float* d_dists, uint64_t* d_counters, void* stream) {
-    if (!h) return fail(DCIH_EINVAL, "dcih_query: null handle");
-    if (dim != h->dim) return fail(DCIH_EINVAL, "dcih_query: dim differs from the index's");
-    if (h->n <= 0) return fail(DCIH_ESTATE, "dcih_query: index is empty");
+// dcih_query.  `fixed` = take every byte of scratch from the
+// device's static array and refuse what does not fit, instead of growing the handle's
+// workspace.
+static int query_impl(dcih_index* h, int dim, int num_queries, const float* d_query,
+                      int num_neighbours, int blind, int num_outer_iterations,
+                      int max_num_candidates, int block_size, int thread_size,
+                      int32_t* d_nn, float* d_dists, uint64_t* d_counters, void* stream,
+                      bool fixed, const char* who) {
+    const std::string me(who);
+    if (!h) return fail(DCIH_EINVAL, me + ": null handle");
+    if (dim != h->dim) return fail(DCIH_EINVAL, me + ": dim differs from the index's");
+    if (h->n <= 0) return fail(DCIH_ESTATE, me + ": index is empty");
     if (num_neighbours <= 0 || num_neighbours > h->n)
-        return fail(DCIH_EINVAL, "dcih_query: num_neighbours must be in [1, num_points]");
+        return fail(DCIH_EINVAL, me + ": num_neighbours must be in [1, num_points]");
     if (num_queries < 0 || (num_queries > 0 && (!d_query || !d_nn || (!blind && !d_dists))))
-        return fail(DCIH_EINVAL, "dcih_query: null buffer");
+        return fail(DCIH_EINVAL, me + ": null buffer");
     // blind: as many candidates per query as the reference's result buffer holds (:782-783)
     const int64_t num_results =
         blind ? std::min<int64_t>(max_num_candidates, num_outer_iterations) : num_neighbours;
     if (num_results <= 0)
-        return fail(DCIH_EINVAL, "dcih_query: blind querying needs positive max_num_candidates and num_outer_iterations");
-    if (thread_size <= 0) return fail(DCIH_EINVAL, "dcih_query: thread_size must be positive");
+        return fail(DCIH_EINVAL, me + ": blind querying needs positive max_num_candidates and num_outer_iterations");
+    if (thread_size <= 0) return fail(DCIH_EINVAL, me + ": thread_size must be positive");
     if (block_size != h->block_size)
-        return fail(DCIH_EINVAL, "dcih_query: block_size differs from the one the index was built with");
+        return fail(DCIH_EINVAL, me + ": block_size differs from the one the index was built with");
     if (num_queries == 0) return DCIH_OK;
     DeviceGuard guard(h->device);
     hipStream_t s = (hipStream_t)stream;
     const int I = num_indices(h);
+    // the scratch of this call: the handle's workspace, grown as needed, or the static array
+    char* ws_base = nullptr;
+    auto get_ws = [&](size_t bytes) -> int {
+        if (!fixed) {
+            const int rc = ensure_ws(h, bytes, s);
+            ws_base = (char*)h->ws;
+            return rc;
+        }
+        return fail(DCIH_EUNSUPPORTED, me + ": no fixed scratch in this build");
+    };
 
     QueryArgs a;
     a.skeys = h->d_skeys; a.sids = h->d_sids; a.inv = h->d_inv; a.lids = h->d_lids; a.data = h->d_data; a.query = d_query;
     a.mode = h->traversal; a.item_list = nullptr; a.item_count = nullptr; a.dense = nullptr;
+    a.xcds = h->xcds; a.q_first = 0; a.q_count = num_queries;
     a.phase_ticks = h->d_phase_ticks;
-    // the hints describe where traversals of one query shape stop; forget them when it changes
+    // the hints describe where traversals of one query shape stop; forget them when it
+    // changes (cleared by a kernel: a memset node is not safe in a captured graph)
     if (h->hint_k != num_neighbours || h->hint_outer != num_outer_iterations ||
         h->hint_T != thread_size || h->hint_maxc != max_num_candidates) {
-        DCIH_HIP(hipMemsetAsync(h->d_stop_hint, 0, (size_t)3 * block_size * sizeof(float), s));
+        const int rc = zero_words64(h->d_stop_hint, (int64_t)(((size_t)3 * block_size * sizeof(float) + 7) / 8), s);
+        if (rc) return rc;
         h->hint_k = num_neighbours; h->hint_outer = num_outer_iterations;
         h->hint_T = thread_size; h->hint_maxc = max_num_candidates;
     }
@@ -390,6 +502,9 @@ int dcih_query(dcih_index* h, int dim, int num_queries, const float* d_query,
     a.counters = (unsigned long long*)d_counters;
     a.out_ids = d_nn; a.out_dists = d_dists;
 
+    if (fixed && num_results > 8192)
+        return fail(DCIH_EUNSUPPORTED, me + ": more than 8192 results per query need the row-per-query "
+                                            "workspace of dcih_query");
     if (num_results > 8192 &&
         (blind || num_neighbours < a.ppb || (num_neighbours == a.ppb && d_counters))) {
         // More results than the top-k tables hold while partitions may still stop early: the
@@ -401,11 +516,11 @@ int dcih_query(dcih_index* h, int dim, int num_queries, const float* d_query,
         const size_t qp_bytes = align_up((size_t)I * chunk * sizeof(float));
         const size_t rank_bytes = align_up(exhaustive_ws_bytes(h->n, chunk));
         const size_t gs_bytes = align_up(query_gscratch_bytes(probe));
-        int rc = ensure_ws(h, qp_bytes + rank_bytes + gs_bytes);
+        int rc = get_ws(qp_bytes + rank_bytes + gs_bytes);
         if (rc) return rc;
-        a.gscratch = gs_bytes ? (uint32_t*)((char*)h->ws + qp_bytes + rank_bytes) : nullptr;
+        a.gscratch = gs_bytes ? (uint32_t*)(ws_base + qp_bytes + rank_bytes) : nullptr;
         mark(h, DCIH_T_TRAVERSE, 0, s);
-        rc = query_dense(a, h->d_dirs, h->ws, chunk, s);
+        rc = query_dense(a, h->d_dirs, ws_base, chunk, s);
         mark(h, DCIH_T_TRAVERSE, 1, s);
         return rc;
     }
@@ -413,8 +528,9 @@ int dcih_query(dcih_index* h, int dim, int num_queries, const float* d_query,
     // max_num_candidates and fewer windows per simple index (at most ppb / T + 3) than
     // num_outer_iterations: the loop then runs every partition dry, as in the reference's own
     // example (3000 points in 100 partitions, 5000 iterations).  Left to pick, the engine
-    // computes that answer directly as well.
-    const bool runs_dry = !blind && h->traversal == 0 && a.ppb < (int64_t)max_num_candidates &&
+    // computes that answer directly as well (not with the fixed scratch, which a million
+    // points per query would overrun: there the traversal kernels give the same neighbours).
+    const bool runs_dry = !blind && !fixed && h->traversal == 0 && a.ppb < (int64_t)max_num_candidates &&
                           a.ppb / thread_size + 4 < (int64_t)num_outer_iterations;
     if (!blind && (num_neighbours > 8192 || runs_dry)) {
         // With more neighbours asked for than a partition holds, no partition can stop early
@@ -424,15 +540,15 @@ int dcih_query(dcih_index* h, int dim, int num_queries, const float* d_query,
         // traversal above.)
         const int chunk = exhaustive_chunk(h->n, num_queries);
         const size_t qp_bytes = d_counters ? align_up((size_t)I * num_queries * sizeof(float)) : 0;
-        int rc = ensure_ws(h, qp_bytes + exhaustive_ws_bytes(h->n, chunk));
+        int rc = get_ws(qp_bytes + exhaustive_ws_bytes(h->n, chunk));
         if (rc) return rc;
         if (d_counters) {
-            rc = project(h->d_dirs, I, d_query, num_queries, dim, (float*)h->ws, s);
+            rc = project(h->d_dirs, I, d_query, num_queries, dim, (float*)ws_base, num_queries, s);
             if (rc) return rc;
-            a.qproj = (float*)h->ws;
+            a.qproj = (float*)ws_base;
         }
         mark(h, DCIH_T_TRAVERSE, 0, s);
-        rc = query_exhaustive(a, (char*)h->ws + qp_bytes, chunk, s);
+        rc = query_exhaustive(a, ws_base + qp_bytes, chunk, s);
         mark(h, DCIH_T_TRAVERSE, 1, s);
         return rc;
     }
@@ -441,9 +557,9 @@ int dcih_query(dcih_index* h, int dim, int num_queries, const float* d_query,
     const size_t part_bytes = align_up(query_part_bytes(a));
     const size_t gs_bytes = align_up(query_gscratch_bytes(a));
     const size_t redo_bytes = align_up((size_t)num_queries * block_size * sizeof(int32_t));
-    int rc = ensure_ws(h, qp_bytes + part_bytes + gs_bytes + redo_bytes + 256);
+    int rc = get_ws(qp_bytes + part_bytes + gs_bytes + redo_bytes + 256);
     if (rc) return rc;
-    char* base = (char*)h->ws;
+    char* base = ws_base;
     float* d_qproj = (float*)base;
     a.qproj = d_qproj;
     a.part = (unsigned long long*)(base + qp_bytes);
@@ -452,7 +568,7 @@ int dcih_query(dcih_index* h, int dim, int num_queries, const float* d_query,
     a.redo_count = (uint32_t*)(base + qp_bytes + part_bytes + gs_bytes + redo_bytes);
 
     mark(h, DCIH_T_QPROJECT, 0, s);
-    rc = project(h->d_dirs, I, d_query, num_queries, dim, d_qproj, s);
+    rc = project(h->d_dirs, I, d_query, num_queries, dim, d_qproj, num_queries, s);
     mark(h, DCIH_T_QPROJECT, 1, s);
     if (rc) return rc;
     hipEvent_t qev[3] = {h->ev[2 * DCIH_T_TRAVERSE], h->ev[2 * DCIH_T_TRAVERSE + 1],
@@ -463,6 +579,31 @@ int dcih_query(dcih_index* h, int dim, int num_queries, const float* d_query,
         h->ev_valid[DCIH_T_TRAVERSE] = h->ev_valid[DCIH_T_MERGE] = true;
     }
     return rc;
+}
+
+int dcih_query(dcih_index* h, int dim, int num_queries, const float* d_query,
+               int num_neighbours, int blind, int num_outer_iterations,
+               int max_num_candidates, int block_size, int thread_size,
+               int32_t* d_nn, float* d_dists, uint64_t* d_counters, void* stream) {
+    return query_impl(h, dim, num_queries, d_query, num_neighbours, blind, num_outer_iterations,
+                      max_num_candidates, block_size, thread_size, d_nn, d_dists, d_counters, stream,
+                      false, "dcih_query");
+}
+
+int64_t dcih_debug_launch_map(int xcds, int block_size, int num_queries, int64_t block,
+                              int* b, int* q, int* queries_per_launch) {
+    if (xcds < 1 || block_size < 1 || num_queries < 1) return -1;
+    const int per_launch = block_queries_per_launch(xcds, block_size, num_queries);
+    if (queries_per_launch) *queries_per_launch = per_launch;
+    if (per_launch < 1) return -1;
+    const int nq = std::min(per_launch, num_queries);
+    const int64_t items = block_items(xcds, block_size, nq);
+    if (b && q && block >= 0 && block < items) {
+        int bb = -1, qq = -1;
+        if (!block_item(block, xcds, block_size, nq, bb, qq)) bb = qq = -1;
+        *b = bb; *q = qq;
+    }
+    return items;
 }
 
 int dcih_set_option(dcih_index* h, int option, int value) {
@@ -551,7 +692,7 @@ int dcih_project(const float* d_dirs, int num_idx, const float* d_rows, int64_t 
                  int dim, float* d_out, void* stream) {
     if (!d_dirs || !d_rows || !d_out || num_idx <= 0 || num_rows < 0 || dim <= 0)
         return fail(DCIH_EINVAL, "dcih_project: bad argument");
-    return project(d_dirs, num_idx, d_rows, num_rows, dim, d_out, (hipStream_t)stream);
+    return project(d_dirs, num_idx, d_rows, num_rows, dim, d_out, num_rows, (hipStream_t)stream);
 }
 
 int dcih_segsort(const float* d_keys, int num_idx, int64_t num_points, int block_size,
@@ -562,7 +703,7 @@ int dcih_segsort(const float* d_keys, int num_idx, int64_t num_points, int block
     const size_t tmp_bytes = segsort_tmp_bytes(num_idx, num_points, block_size);
     void* d_tmp = nullptr;
     if (tmp_bytes) DCIH_HIP(hipMalloc(&d_tmp, tmp_bytes));
-    const int rc = segsort(d_keys, num_idx, num_points, block_size, d_skeys, d_sids, nullptr, nullptr, d_tmp, s);
+    const int rc = segsort(d_keys, num_points, num_idx, num_points, block_size, d_skeys, d_sids, nullptr, nullptr, d_tmp, s);
     if (d_tmp) {
         (void)hipStreamSynchronize(s);
         (void)hipFree(d_tmp);

@@ -160,7 +160,7 @@ int rank_rows(void* ws, int chunk, int rows, int64_t N, int k, bool inf_is_empty
     float* d_sorted = (float*)(base + align256(cells * 4));
     int32_t* d_sids = (int32_t*)(base + 2 * align256(cells * 4));
     void* d_tmp = segsort_tmp_bytes(chunk, N, 1) ? (void*)(base + 3 * align256(cells * 4)) : nullptr;
-    const int rc = segsort(d_in, rows, N, 1, d_sorted, d_sids, nullptr, nullptr, d_tmp, s);
+    const int rc = segsort(d_in, N, rows, N, 1, d_sorted, d_sids, nullptr, nullptr, d_tmp, s);
     if (rc) return rc;
     hipLaunchKernelGGL(take_columns_kernel, dim3((unsigned)min(1024, (k + 255) / 256), (unsigned)rows),
                        dim3(256), 0, s, d_sorted, d_sids, N, k, inf_is_empty ? 1 : 0, out_ids, out_vals);

@@ -6,19 +6,21 @@
 
 namespace dcih {
 
-// out[r][c] = sum_k rows[c][k] * dirs[r][k]; out is [num_dirs][num_rows].
+// out[r][c] = sum_k rows[c][k] * dirs[r][k]; row r of out starts at d_out + r * out_stride
+// (out_stride >= num_rows).
 int project(const float* d_dirs, int num_dirs, const float* d_rows, int64_t num_rows,
-            int dim, float* d_out, hipStream_t s);
+            int dim, float* d_out, int64_t out_stride, hipStream_t s);
 
-// Sorts every (simple index, partition) slice of keys [num_indices][n] by
-// (key, id).  d_tmp is scratch of segsort_tmp_bytes() bytes (may be null when
+// Sorts every (simple index, partition) slice of the keys by (key, id); the keys of
+// index i start at d_keys + i * key_stride (key_stride >= n), the outputs are
+// [num_indices][n].  d_tmp is scratch of segsort_tmp_bytes() bytes (may be null when
 // that is 0).
 size_t segsort_tmp_bytes(int num_indices, int64_t n, int block_size);
 // d_inv: null, or [num_indices][n] receiving each point's position inside its
 // sorted slice (the inverse of d_sids) as a 16-bit value.  d_lids: null, or [num_indices][n]
 // receiving the ids relative to their partition's first point as 16-bit values
 // (only meaningful when a partition holds at most 65536 points).
-int segsort(const float* d_keys, int num_indices, int64_t n, int block_size,
+int segsort(const float* d_keys, int64_t key_stride, int num_indices, int64_t n, int block_size,
             float* d_skeys, int32_t* d_sids, uint16_t* d_inv, uint16_t* d_lids, void* d_tmp,
             hipStream_t s);
 
@@ -50,11 +52,56 @@ struct QueryArgs {
     float* stop_hint;        // null, or [3][B] per partition: running averages of the stop step and of the promotions at the stop, stops seen
     unsigned long long* phase_ticks;  // null, or 16 accumulators for the batch kernel's phases
     int mode;                // 0 = pick, 1 = step-by-step kernel, 2 = batch kernel
+    int xcds;                // accelerator dies of the device (each has an L2 of its own)
+    int q_first, q_count;    // batch kernel: the queries one launch covers
     int32_t* out_ids;        // [nq][k]
     float* out_dists;        // [nq][k]; blind: null, or the promoting steps as floats
     float* dense;            // null, or [nq][N]: the step-by-step kernel stores every candidate's score here instead of keeping a top-k
 };
+// Work order of the batch kernel.  Workgroups go to the XCDs round-robin by their
+// number and every XCD has an L2 of its own, so XCD x is given the partitions x,
+// x + X, ... and works through them one after the other, all queries of a
+// partition before the next: the workgroups an XCD runs at any moment share one
+// partition's slices.  The B mod X partitions that do not fill a round are spread
+// over all X dies as equal runs of the (partition, query) list, so no die idles.
+// block_items = workgroups one launch over nq queries needs; block_item maps a
+// workgroup to its partition b and query q (false: nothing to do).
+__host__ __device__ inline int64_t block_items(int X, int B, int nq) {
+    const int full = B / X, rest = B - full * X;
+    return (int64_t)X * ((int64_t)full * nq + ((int64_t)rest * nq + X - 1) / X);
+}
+__host__ __device__ inline bool block_item(int64_t block, int X, int B, int nq, int& b, int& q) {
+    const int xcd = (int)(block % X);
+    const int64_t seq = block / X;
+    const int full = B / X, rest = B - full * X;
+    const int64_t full_items = (int64_t)full * nq;
+    if (seq < full_items) {
+        b = xcd + X * (int)(seq / nq);
+        q = (int)(seq % nq);
+        return true;
+    }
+    const int64_t run = ((int64_t)rest * nq + X - 1) / X;
+    const int64_t e = (seq - full_items) + (int64_t)xcd * run;
+    if (seq - full_items >= run || e >= (int64_t)rest * nq) return false;
+    b = X * full + (int)(e / nq);
+    q = (int)(e % nq);
+    return true;
+}
+// Queries one launch of the batch kernel may cover: a launch is limited to 2^32 - 1
+// threads in all (256 per workgroup).
+__host__ __device__ inline int block_queries_per_launch(int X, int B, int nq) {
+    const int64_t max_items = 0xffffffffLL / 256;
+    const int64_t per_query = (int64_t)B + X;          // upper bound of block_items / nq
+    const int64_t fit = max_items / per_query;
+    return (int)(fit < 1 ? 0 : (fit < nq ? fit : nq));
+}
+// Workgroups of the step-by-step kernel: it strides over its items, and a launch is
+// limited to 2^32 - 1 threads in all (64 per workgroup).
+__host__ __device__ inline int64_t step_grid_cap() { return (int64_t)1 << 20; }
+
 size_t query_part_bytes(const QueryArgs& a);
+// Clears n 64-bit words with a kernel (a memset node is not safe in a captured graph).
+int zero_words64(void* d_p, int64_t n, hipStream_t s);
 // Bytes of global counter scratch the traversal needs (0 when LDS suffices).
 size_t query_gscratch_bytes(const QueryArgs& a);
 // Batch traversal (traverse_block.hip): whether the shape fits its fixed LDS

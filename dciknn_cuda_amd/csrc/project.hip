@@ -37,7 +37,7 @@ constexpr int kProjLoads = kProjRows / kProjRpp;  // 16-byte loads per lane and 
 template <int RT>
 __global__ __launch_bounds__(kProjRows) void project_kernel(
     const float* __restrict__ dirs, int r0, const float* __restrict__ rows,
-    int64_t num_rows, int dim, float* __restrict__ out) {
+    int64_t num_rows, int dim, float* __restrict__ out, int64_t out_stride) {
     __shared__ float tile[kProjRows * kProjStride];
     const int tid = threadIdx.x;
     const int64_t row0 = min((int64_t)blockIdx.x * kProjRows, num_rows - kProjRows);
@@ -146,14 +146,14 @@ __global__ __launch_bounds__(kProjRows) void project_kernel(
     }
 #pragma unroll
     for (int r = 0; r < RT; r++)
-        out[(int64_t)(r0 + r) * num_rows + row0 + tid] = acc[r] + 0.0f;  // -0.0 -> +0.0
+        out[(int64_t)(r0 + r) * out_stride + row0 + tid] = acc[r] + 0.0f;  // -0.0 -> +0.0
 }
 
 // Any shape: one row per thread straight from global memory, same FMA order.
 template <int RT>
 __global__ __launch_bounds__(256) void project_generic_kernel(
     const float* __restrict__ dirs, int r0, const float* __restrict__ rows,
-    int64_t num_rows, int dim, float* __restrict__ out) {
+    int64_t num_rows, int dim, float* __restrict__ out, int64_t out_stride) {
     const int64_t row = (int64_t)blockIdx.x * 256 + threadIdx.x;
     if (row >= num_rows) return;
     float acc[RT];
@@ -168,44 +168,45 @@ __global__ __launch_bounds__(256) void project_generic_kernel(
         for (int r = 0; r < RT; r++) acc[r] = __builtin_fmaf(v, dk[(int64_t)r * dim + k], acc[r]);
     }
 #pragma unroll
-    for (int r = 0; r < RT; r++) out[(int64_t)(r0 + r) * num_rows + row] = acc[r] + 0.0f;
+    for (int r = 0; r < RT; r++) out[(int64_t)(r0 + r) * out_stride + row] = acc[r] + 0.0f;
 }
 
 template <int RT>
 static void launch_project(const float* dirs, int r0, const float* rows,
-                           int64_t num_rows, int dim, float* out, hipStream_t s) {
+                           int64_t num_rows, int dim, float* out, int64_t out_stride, hipStream_t s) {
     // float4 loads need 16-byte aligned row starts
     const bool fast = (dim & 3) == 0 && (reinterpret_cast<uintptr_t>(rows) & 15) == 0 &&
                       num_rows >= kProjRows;
     if (fast) {
         const int64_t blocks = (num_rows + kProjRows - 1) / kProjRows;
         hipLaunchKernelGGL(project_kernel<RT>, dim3((unsigned)blocks), dim3(kProjRows), 0, s,
-                           dirs, r0, rows, num_rows, dim, out);
+                           dirs, r0, rows, num_rows, dim, out, out_stride);
     } else {
         const int64_t blocks = (num_rows + 255) / 256;
         hipLaunchKernelGGL(project_generic_kernel<RT>, dim3((unsigned)blocks), dim3(256), 0, s,
-                           dirs, r0, rows, num_rows, dim, out);
+                           dirs, r0, rows, num_rows, dim, out, out_stride);
     }
 }
 
 template <int RT>
 static void dispatch_tail(int rt, const float* dirs, int r0, const float* rows,
-                          int64_t num_rows, int dim, float* out, hipStream_t s) {
+                          int64_t num_rows, int dim, float* out, int64_t out_stride, hipStream_t s) {
     if constexpr (RT >= 1) {
-        if (rt == RT) launch_project<RT>(dirs, r0, rows, num_rows, dim, out, s);
-        else dispatch_tail<RT - 1>(rt, dirs, r0, rows, num_rows, dim, out, s);
+        if (rt == RT) launch_project<RT>(dirs, r0, rows, num_rows, dim, out, out_stride, s);
+        else dispatch_tail<RT - 1>(rt, dirs, r0, rows, num_rows, dim, out, out_stride, s);
     }
 }
 
 int project(const float* d_dirs, int num_dirs, const float* d_rows, int64_t num_rows,
-            int dim, float* d_out, hipStream_t s) {
+            int dim, float* d_out, int64_t out_stride, hipStream_t s) {
     if (num_rows <= 0 || num_dirs <= 0) return 0;
+    if (out_stride < num_rows) return fail(-1, "project: output rows overlap");
     if ((num_rows + kProjRows - 1) / kProjRows > 0x7fffffffLL)
         return fail(-1, "project: too many rows for one launch");
     int r0 = 0;
     while (num_dirs - r0 > 0) {
         const int rt = min(32, num_dirs - r0);
-        dispatch_tail<32>(rt, d_dirs, r0, d_rows, num_rows, dim, d_out, s);
+        dispatch_tail<32>(rt, d_dirs, r0, d_rows, num_rows, dim, d_out, out_stride, s);
         r0 += rt;
     }
     DCIH_HIP(hipGetLastError());

@@ -334,13 +334,21 @@ static int allow_full_lds() {
     });
 }
 
+int zero_words64(void* d_p, int64_t n, hipStream_t s) {
+    if (n <= 0) return 0;
+    hipLaunchKernelGGL(zero_u64_kernel, dim3((unsigned)max((int64_t)1, min((int64_t)1024, (n + 255) / 256))),
+                       dim3(256), 0, s, (unsigned long long*)d_p, n, (uint32_t*)nullptr);
+    DCIH_HIP(hipGetLastError());
+    return 0;
+}
+
 size_t query_part_bytes(const QueryArgs& a) {
     return (size_t)a.nq * a.B * a.kcap * sizeof(unsigned long long);
 }
 
 static int64_t traverse_grid(const QueryArgs& a, const Layout& y) {
     const int64_t items = (int64_t)a.nq * a.B;
-    if (y.lds_counters) return min(items, (int64_t)0x7fffffff);
+    if (y.lds_counters) return min(items, step_grid_cap());   // the kernel strides over its items
     return min(items, (int64_t)kMaxSlots);
 }
 
@@ -432,7 +440,7 @@ int query_dense(const QueryArgs& a_in, const float* d_dirs, void* ws, int chunk,
         a.item_list = nullptr;
         a.item_count = nullptr;
         a.dense = rank_rows_input(ws_rank);
-        int rc = project(d_dirs, I, a.query, a.nq, a.dim, d_qproj, s);
+        int rc = project(d_dirs, I, a.query, a.nq, a.dim, d_qproj, a.nq, s);
         if (rc) return rc;
         rc = fill_rows(a.dense, (int64_t)a.nq * a.N, __builtin_inff(), s);
         if (rc) return rc;

@@ -22,6 +22,7 @@ constexpr int kMergeItems = 8;
 constexpr int kMergeChunk = kMergeThreads * kMergeItems;  // divides kTileCap
 
 struct SegGeom {
+    int64_t kstride;  // distance between the unsorted key rows of two indices (>= n)
     int64_t n;        // points
     int64_t ppb;      // points per partition
     int B;            // partitions
@@ -53,9 +54,10 @@ __global__ void segsort_tile_kernel(const float* __restrict__ keys, SegGeom g,
     if (nseg <= 0 || t0 >= nseg) return;
     const int m = (int)min((int64_t)kTileCap, nseg - t0);
     const int64_t base = i * g.n + off + t0;
+    const int64_t kbase = i * g.kstride + off + t0;
 
     for (int j = threadIdx.x; j < np2; j += blockDim.x)
-        s[j] = j < m ? pack_key(keys[base + j], (uint32_t)(t0 + j)) : ~0ull;
+        s[j] = j < m ? pack_key(keys[kbase + j], (uint32_t)(t0 + j)) : ~0ull;
     bitonic_sort_u64(s, np2);
     for (int j = threadIdx.x; j < m; j += blockDim.x) {
         const unsigned long long w = s[j];
@@ -138,6 +140,7 @@ __global__ __launch_bounds__(kRadixThreads, (kRadixThreads == 256 && IPT > 45) ?
     const int n = (int)(packed ? min(nseg, (int64_t)g.tile_size) : nseg);
     if (n <= 0) return;
     const int64_t base = i * g.n + off + t0;
+    const int64_t kbase = i * g.kstride + off + t0;
 
     if (tid < 2) misc[32 + tid] = tid ? 0xffffffffu : 0u;        // OR / AND of all keys
     uint32_t k[IPT], rp[IPT];      // rp: id in the low half, rank / position in the high half
@@ -146,7 +149,7 @@ __global__ __launch_bounds__(kRadixThreads, (kRadixThreads == 256 && IPT > 45) ?
 #pragma unroll
     for (int r = 0; r < IPT; r++) {
         const int j = min(r * kRadixThreads + tid, n - 1);       // unconditional: no branch per load
-        k[r] = __builtin_bit_cast(uint32_t, keys[base + j]);
+        k[r] = __builtin_bit_cast(uint32_t, keys[kbase + j]);
     }
 #pragma unroll
     for (int r = 0; r < IPT; r++) {
@@ -435,11 +438,13 @@ static int next_pow2(int v) {
     return p;
 }
 
-int segsort(const float* d_keys, int num_indices, int64_t n, int block_size,
+int segsort(const float* d_keys, int64_t key_stride, int num_indices, int64_t n, int block_size,
             float* d_skeys, int32_t* d_sids, uint16_t* d_inv, uint16_t* d_lids, void* d_tmp,
             hipStream_t s) {
     if (n <= 0) return 0;
+    if (key_stride < n) return fail(-1, "segsort: key rows overlap");
     SegGeom g;
+    g.kstride = key_stride;
     g.n = n;
     g.B = block_size;
     g.ppb = (n + block_size - 1) / block_size;

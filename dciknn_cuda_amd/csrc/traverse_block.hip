@@ -39,7 +39,6 @@ namespace dcih {
 namespace {
 
 constexpr int kMaxEpochs = 100000;
-constexpr int kXcds = 8;             // accelerator dies of an MI355X, each with its own L2
 constexpr uint32_t kInfBits = 0x7f800000u;
 
 enum Misc {   // 32-bit scalars shared by the workgroup; kStreamedLo must stay 8-byte aligned
@@ -250,16 +249,11 @@ __global__ __launch_bounds__(NT, MINW) void traverse_block_kernel(QueryArgs a, B
     const int I = a.M * a.L;
     const int S = 2 * I;                       // streams
 
-    // Workgroups go to the XCDs round-robin by their number, and every XCD has an L2
-    // of its own.  XCD x gets the partitions x, x + 8, ... and works through them one
-    // after the other, all queries of a partition before the next: the workgroups an
-    // XCD runs at any moment share one partition's slices (a few MB), which then live
-    // in that L2 instead of being fetched again by every query.
-    const int xcd = (int)(blockIdx.x % kXcds);
-    const int64_t seq = blockIdx.x / kXcds;
-    const int b = xcd + kXcds * (int)(seq / a.nq);
-    const int qi = (int)(seq % a.nq);
-    if (b >= a.B) return;                      // this XCD has one partition fewer than others
+    // which (partition, query) this workgroup works on: see block_item (one partition's
+    // slices stay in the L2 of the XCD that works through its queries)
+    int b, qi;
+    if (!block_item((int64_t)blockIdx.x, a.xcds, a.B, a.q_count, b, qi)) return;
+    qi += a.q_first;
     const int64_t item = (int64_t)qi * a.B + b;
     const int64_t off = (int64_t)b * a.ppb;
     const int n = (int)min(a.N - off, a.ppb);
@@ -1061,14 +1055,21 @@ bool block_traversal_supported(const QueryArgs& a, size_t* lds_bytes) {
     if (a.ppb >= (1 << 25)) return false;
     if ((int64_t)a.L * (a.ppb + 2 * (int64_t)a.T) >= 0x7fffffffLL) return false;   // steps fit 32 bits
     if ((int64_t)a.ppb + 2 * (int64_t)a.T >= 0x7fffffffLL) return false;
-    if ((int64_t)a.nq * (a.B + kXcds) > 0x7fffffffLL) return false;
+    if (a.xcds < 1 || block_queries_per_launch(a.xcds, a.B, a.nq) < 1) return false;
     return y.lds_bytes <= 160 * 1024 - 512;
 }
 
-int query_block(const QueryArgs& a, hipStream_t s) {
-    const BlockLayout y = make_block_layout(a);
-    const int64_t items = (int64_t)a.nq * kXcds * ((a.B + kXcds - 1) / kXcds);
+int query_block(const QueryArgs& a_in, hipStream_t s) {
+    const BlockLayout y = make_block_layout(a_in);
     const int fit = (int)(160 * 1024 / y.lds_bytes);      // workgroups per CU by LDS
+    // as many queries per launch as the launch limit allows (nearly always all of them)
+    const int per_launch = block_queries_per_launch(a_in.xcds, a_in.B, a_in.nq);
+    if (per_launch < 1) return fail(-4, "query: block_size too large for the batch traversal kernel");
+    for (int q0 = 0; q0 < a_in.nq; q0 += per_launch) {
+        QueryArgs a = a_in;
+        a.q_first = q0;
+        a.q_count = min(per_launch, a_in.nq - q0);
+        const int64_t items = block_items(a.xcds, a.B, a.q_count);
 #define DCIH_LAUNCH(CB, MW)                                                                        \
     do {                                                                                           \
         static DeviceOnce once;                                                                    \
@@ -1081,10 +1082,11 @@ int query_block(const QueryArgs& a, hipStream_t s) {
         hipLaunchKernelGGL((traverse_block_kernel<kBlockThreads, CB, MW>), dim3((unsigned)items),  \
                            dim3(kBlockThreads), y.lds_bytes, s, a, y);                             \
     } while (0)
-    if (y.cbits == 4) { if (fit >= 6) DCIH_LAUNCH(4, 6); else if (fit >= 5) DCIH_LAUNCH(4, 5); else if (fit == 4) DCIH_LAUNCH(4, 4); else DCIH_LAUNCH(4, 3); }
-    else              { if (fit >= 6) DCIH_LAUNCH(8, 6); else if (fit >= 5) DCIH_LAUNCH(8, 5); else if (fit == 4) DCIH_LAUNCH(8, 4); else DCIH_LAUNCH(8, 3); }
+        if (y.cbits == 4) { if (fit >= 6) DCIH_LAUNCH(4, 6); else if (fit >= 5) DCIH_LAUNCH(4, 5); else if (fit == 4) DCIH_LAUNCH(4, 4); else DCIH_LAUNCH(4, 3); }
+        else              { if (fit >= 6) DCIH_LAUNCH(8, 6); else if (fit >= 5) DCIH_LAUNCH(8, 5); else if (fit == 4) DCIH_LAUNCH(8, 4); else DCIH_LAUNCH(8, 3); }
 #undef DCIH_LAUNCH
-    DCIH_HIP(hipGetLastError());
+        DCIH_HIP(hipGetLastError());
+    }
     return 0;
 }
 

@@ -107,9 +107,12 @@ int dcih_add(dcih_index* h, int dim, int64_t num_points, const float* d_data,
  * exactly the index dcih_add would build over all rows given so far, in the order
  * given (ids continue where the previous call stopped).  Unlike dcih_add the rows
  * are COPIED into a buffer the index owns, so d_data may be released after the
- * call; rows of an earlier dcih_add are copied as well.  The partition boundaries
- * depend on the total, so every slice is projected and sorted again.  Synchronises
- * the stream.
+ * call; rows of an earlier dcih_add are copied as well.  The index also keeps the
+ * unsorted projections of its rows, so only the new rows are projected; the
+ * partition boundaries depend on the total, so every slice is formed again.  The
+ * next index is built beside the current one (twice the index's memory while the
+ * call runs): if the call fails, for lack of memory or otherwise, the index is
+ * what it was before.  Synchronises the stream.
  */
 int dcih_append(dcih_index* h, int dim, int64_t num_points, const float* d_data,
                 int block_size, int thread_size, void* stream);
@@ -216,12 +219,25 @@ int dcih_free(dcih_index* h);
  *   dcih_project : out[r][c] = sum_k d_rows[c][k] * d_dirs[r][k]  (the SGEMM at
  *                  src/util_kernel.cu:76 as used at src/dci_cuda_kernel.cu:167-169)
  *   dcih_segsort : copy_to_indices + sort_indices
- *                  (src/dci_cuda_kernel.cu:113-146), ties by id
+ *                  (src/dci_cuda_kernel.cu:113-146), ties by id; -0.0 compares
+ *                  equal to +0.0 (so they tie on the id) and is stored as +0.0
  */
 int dcih_project(const float* d_dirs, int num_indices, const float* d_rows,
                  int64_t num_rows, int dim, float* d_out, void* stream);
 int dcih_segsort(const float* d_keys, int num_indices, int64_t num_points,
                  int block_size, float* d_skeys, int32_t* d_sids, void* stream);
+
+/*
+ * Launch geometry of the batch traversal kernel (no counterpart in the reference;
+ * pure host arithmetic, no GPU needed): with `xcds` dies, block_size partitions and
+ * num_queries queries, returns the number of workgroups one launch starts, or -1
+ * if the shape cannot be launched; if b and q are not NULL and 0 <= block < that
+ * number, *b / *q receive the partition and query workgroup `block` works on, or
+ * -1 / -1 if it has nothing to do.  *queries_per_launch (if not NULL) receives how
+ * many queries one launch may cover (a launch is limited to 2^32 - 1 threads).
+ */
+int64_t dcih_debug_launch_map(int xcds, int block_size, int num_queries, int64_t block,
+                              int* b, int* q, int* queries_per_launch);
 
 #ifdef __cplusplus
 }

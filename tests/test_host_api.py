@@ -46,6 +46,47 @@ def test_null_and_bad_arguments_return_status_codes():
         _capi.check(lib.dcih_clear(None))
 
 
+@pytest.mark.parametrize("xcds,B,nq", [(8, 56, 10), (8, 100, 7), (8, 3, 5), (8, 1, 1), (8, 9, 16),
+                                       (4, 10, 3), (1, 5, 4), (8, 13, 1), (8, 8, 3)])
+def test_batch_kernel_launch_map_covers_every_item_once(xcds, B, nq):
+    """Every (partition, query) pair belongs to exactly one workgroup, workgroup w runs on
+    die w mod xcds, a die works through one partition's queries before the next partition's,
+    and the dies' shares differ by at most one run of the leftover partitions."""
+    from dciknn_cuda_amd import _capi
+    lib = _capi.lib()
+    b, q, per = ctypes.c_int(), ctypes.c_int(), ctypes.c_int()
+    items = lib.dcih_debug_launch_map(xcds, B, nq, -1, None, None, ctypes.byref(per))
+    assert per.value == nq and items >= B * nq and items * 256 < 2 ** 32
+    seen = {}
+    load = [0] * xcds
+    order = [[] for _ in range(xcds)]
+    for w in range(items):
+        assert lib.dcih_debug_launch_map(xcds, B, nq, w, ctypes.byref(b), ctypes.byref(q), None) == items
+        if b.value < 0:
+            assert q.value < 0
+            continue
+        assert 0 <= b.value < B and 0 <= q.value < nq
+        assert (b.value, q.value) not in seen
+        seen[(b.value, q.value)] = w
+        load[w % xcds] += 1
+        order[w % xcds].append(b.value)
+    assert len(seen) == B * nq
+    assert max(load) - min(load) <= -(-((B % xcds) * nq) // xcds)
+    for o in order:      # partitions appear in runs: never back to an earlier one
+        assert o == sorted(o)
+
+
+def test_batch_kernel_launch_is_chunked_below_the_thread_limit():
+    from dciknn_cuda_amd import _capi
+    lib = _capi.lib()
+    per = ctypes.c_int()
+    # 10000 queries x 4000 partitions would be 40 M workgroups of 256 threads: over 2^32 threads
+    items = lib.dcih_debug_launch_map(8, 4000, 10000, -1, None, None, ctypes.byref(per))
+    assert 0 < per.value < 10000
+    assert items * 256 < 2 ** 32
+    assert lib.dcih_debug_launch_map(8, 2 ** 30, 10, -1, None, None, ctypes.byref(per)) == -1
+
+
 def test_extension_module_exports_the_reference_names():
     """The seven functions dciknn_cuda/core.py:19 imports, plus the handle accessor."""
     from dciknn_cuda_amd import _dci_cuda
