@@ -13,6 +13,7 @@ NUM_COUNTERS = 4
 CTR_VISITED, CTR_CANDIDATES, CTR_PROBES, CTR_STEPS = range(4)
 OPT_TRAVERSAL = 0
 TRAVERSAL_AUTO, TRAVERSAL_STEP, TRAVERSAL_BATCH = 0, 1, 2
+NOALLOC_SCRATCH_BYTES = 32 << 20
 NUM_TIMERS = 5
 T_PROJECT, T_SEGSORT, T_QPROJECT, T_TRAVERSE, T_MERGE = range(5)
 
@@ -32,6 +33,9 @@ SIGNATURES = {
     "dcih_query": (_c.c_int, [_c.c_void_p, _c.c_int, _c.c_int, _c.c_void_p, _c.c_int,
                               _c.c_int, _c.c_int, _c.c_int, _c.c_int, _c.c_int,
                               _c.c_void_p, _c.c_void_p, _c.c_void_p, _c.c_void_p]),
+    "dcih_query_noalloc": (_c.c_int, [_c.c_void_p, _c.c_int, _c.c_int, _c.c_void_p, _c.c_int,
+                                      _c.c_int, _c.c_int, _c.c_int, _c.c_int, _c.c_int,
+                                      _c.c_void_p, _c.c_void_p, _c.c_void_p, _c.c_void_p]),
     "dcih_debug_launch_map": (_c.c_int64, [_c.c_int, _c.c_int, _c.c_int, _c.c_int64,
                                            _c.POINTER(_c.c_int), _c.POINTER(_c.c_int),
                                            _c.POINTER(_c.c_int)]),

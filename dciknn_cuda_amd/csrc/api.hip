@@ -77,6 +77,39 @@ struct DeviceGuard {
 
 using namespace dcih;
 
+// Scratch of dcih_query_noalloc: part of the code object, so every device the library
+// runs on holds its own copy from the moment the library is loaded there until the
+// process ends.  Host code never uses this name as an address (on the host it is only a
+// stand-in for the symbol): dcih_create asks the runtime where the array lives on its
+// device and keeps that pointer.  (The host code's use of the name below is what gives the
+// device symbol external linkage, which the runtime's lookup by name needs: a `used`
+// attribute would keep it local to the code object and the lookup would abort.)
+constexpr size_t kScratchBytes = DCIH_NOALLOC_SCRATCH_BYTES;
+static __device__ __align__(256) unsigned char scratch[kScratchBytes];
+
+namespace {
+constexpr int kMaxDevices = 64;
+std::mutex g_scratch_mu;
+void* g_scratch_ptr[kMaxDevices] = {};
+
+// Device address of `scratch` on `device`, which must be the current device.
+int resolve_scratch(int device) {
+    if (device < 0 || device >= kMaxDevices) return fail(DCIH_EINVAL, "device number out of range");
+    std::lock_guard<std::mutex> lock(g_scratch_mu);
+    if (g_scratch_ptr[device]) return 0;
+    void* ptr = nullptr;
+    DCIH_HIP(hipGetSymbolAddress(&ptr, HIP_SYMBOL(scratch)));
+    if (!ptr) return fail(DCIH_EHIP, "hipGetSymbolAddress returned no address for the scratch array");
+    g_scratch_ptr[device] = ptr;
+    return 0;
+}
+
+void* scratch_of(int device) {
+    std::lock_guard<std::mutex> lock(g_scratch_mu);
+    return device >= 0 && device < kMaxDevices ? g_scratch_ptr[device] : nullptr;
+}
+}  // namespace
+
 struct dcih_index {
     int dim = 0, M = 0, L = 0, device = 0;
     int xcds = 8;                       // accelerator dies of the device
@@ -259,6 +292,7 @@ int dcih_create(int dim, int num_comp_indices, int num_simp_indices, int device,
             h->xcds = xcds;
         (void)hipGetLastError();
     }
+    if (const int rc_s = resolve_scratch(device)) { delete h; return rc_s; }
     const size_t bytes = (size_t)num_indices(h) * dim * sizeof(float);
     if (hipMalloc(&h->d_dirs, bytes) != hipSuccess) {
         delete h;
@@ -436,7 +470,7 @@ int dcih_append(dcih_index* h, int dim, int64_t num_points, const float* d_data,
     return DCIH_OK;
 }
 
-// dcih_query.  `fixed` = take every byte of scratch from the
+// dcih_query and dcih_query_noalloc.  `fixed` = take every byte of scratch from the
 // device's static array and refuse what does not fit, instead of growing the handle's
 // workspace.
 static int query_impl(dcih_index* h, int dim, int num_queries, const float* d_query,
@@ -472,7 +506,13 @@ static int query_impl(dcih_index* h, int dim, int num_queries, const float* d_qu
             ws_base = (char*)h->ws;
             return rc;
         }
-        return fail(DCIH_EUNSUPPORTED, me + ": no fixed scratch in this build");
+        ws_base = (char*)scratch_of(h->device);
+        if (!ws_base) return fail(DCIH_ESTATE, me + ": the scratch array of this device was not located");
+        if (bytes > kScratchBytes)
+            return fail(DCIH_EINVAL, me + ": this call needs " + std::to_string(bytes) +
+                                     " bytes of scratch and the fixed array holds " +
+                                     std::to_string(kScratchBytes) + "; pass fewer queries per call");
+        return 0;
     };
 
     QueryArgs a;
@@ -588,6 +628,15 @@ int dcih_query(dcih_index* h, int dim, int num_queries, const float* d_query,
     return query_impl(h, dim, num_queries, d_query, num_neighbours, blind, num_outer_iterations,
                       max_num_candidates, block_size, thread_size, d_nn, d_dists, d_counters, stream,
                       false, "dcih_query");
+}
+
+int dcih_query_noalloc(dcih_index* h, int dim, int num_queries, const float* d_query,
+                       int num_neighbours, int blind, int num_outer_iterations,
+                       int max_num_candidates, int block_size, int thread_size,
+                       int32_t* d_nn, float* d_dists, uint64_t* d_counters, void* stream) {
+    return query_impl(h, dim, num_queries, d_query, num_neighbours, blind, num_outer_iterations,
+                      max_num_candidates, block_size, thread_size, d_nn, d_dists, d_counters, stream,
+                      true, "dcih_query_noalloc");
 }
 
 int64_t dcih_debug_launch_map(int xcds, int block_size, int num_queries, int64_t block,

@@ -161,6 +161,30 @@ int dcih_query(dcih_index* h, int dim, int num_queries, const float* d_query,
                int32_t* d_nn, float* d_dists, uint64_t* d_counters, void* stream);
 
 /*
+ * dcih_query for callers that cannot allocate device memory: code under HIP graph
+ * capture, tight serving loops, harnesses that forbid hipMalloc.  It has no
+ * counterpart in the reference.  Same arguments, same results and same kernels as
+ * dcih_query, but every byte of scratch (query projections, per-partition result
+ * lists, hand-over list between the two traversal kernels, global visit counters
+ * of partitions too large for on-chip memory) comes from one array of
+ * DCIH_NOALLOC_SCRATCH_BYTES that is part of the library's code object, so each
+ * GPU the library runs on holds one such array until the process ends.  The call
+ * makes no hipMalloc / hipFree and uses no allocating library routine.  A call
+ * that needs more scratch than the array holds returns DCIH_EINVAL and says how
+ * much it needs (the need grows with num_queries * block_size *
+ * min(num_neighbours, points per partition): pass fewer queries per call); more
+ * than 8192 results per query return DCIH_EUNSUPPORTED.  All calls on one GPU
+ * share that GPU's array: calls that overlap in time on the same GPU (different
+ * streams or threads) race and must be serialised by the caller; a call that
+ * follows another on the same stream is safe, it overwrites what it uses.
+ */
+#define DCIH_NOALLOC_SCRATCH_BYTES (32u << 20)
+int dcih_query_noalloc(dcih_index* h, int dim, int num_queries, const float* d_query,
+                       int num_neighbours, int blind, int num_outer_iterations,
+                       int max_num_candidates, int block_size, int thread_size,
+                       int32_t* d_nn, float* d_dists, uint64_t* d_counters, void* stream);
+
+/*
  * Inspection of the built index (no counterpart in the reference besides the
  * debug printer dci_dump, src/dci_cuda_kernel.cu:901-912).  Copies the sorted
  * projections and point ids, both [num_indices][num_points], to host buffers;

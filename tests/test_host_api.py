@@ -36,6 +36,7 @@ def test_null_and_bad_arguments_return_status_codes():
     assert lib.dcih_add(None, 4, 10, None, 1, 1, None) == -1
     assert b"null handle" in lib.dcih_last_error()
     assert lib.dcih_query(None, 4, 1, None, 1, 0, 1, 10, 1, 1, None, None, None, None) == -1
+    assert lib.dcih_query_noalloc(None, 4, 1, None, 1, 0, 1, 10, 1, 1, None, None, None, None) == -1
     assert lib.dcih_create(0, 1, 1, 0, 0, ctypes.byref(ctypes.c_void_p())) == -1
     assert lib.dcih_create(4, 1, 1, 0, 0, None) == -1
     assert lib.dcih_project(None, 1, None, 1, 1, None, None) == -1

@@ -1,0 +1,77 @@
+"""dcih_query_noalloc (all scratch from the library's fixed device array, no
+allocation) against dcih_query on the same index and queries: identical ids,
+distances and counters, on two calls in a row, the second with a smaller input,
+plus its size limit."""
+import numpy as np
+import pytest
+import torch
+
+pytestmark = pytest.mark.gpu
+
+
+def _call(dci, fn, Q, k, outer, B, T, blind=0, counters=True):
+    from dciknn_cuda_amd import _capi
+    nq = Q.shape[0]
+    width = min(10 * k, outer) if blind else k
+    ids = torch.full((nq, width), -7, dtype=torch.int32, device="cuda")
+    dists = torch.full((nq, width), -7.0, dtype=torch.float32, device="cuda")
+    ctr = torch.full((nq, 4), -7, dtype=torch.int64, device="cuda") if counters else None
+    rc = fn(dci._dci_inst, Q.shape[1], nq, Q.data_ptr(), k, blind, outer, 10 * k, B, T,
+            ids.data_ptr(), dists.data_ptr(), ctr.data_ptr() if counters else None,
+            torch.cuda.current_stream().cuda_stream)
+    _capi.check(rc)
+    torch.cuda.synchronize()
+    return ids, dists, ctr
+
+
+@pytest.mark.parametrize("traversal", ["auto", "step"])
+def test_noalloc_equals_query_twice_second_smaller(gpu, traversal):
+    g = torch.Generator().manual_seed(21)
+    dim, M, L, B, T, k, outer = 32, 2, 6, 12, 3, 9, 40
+    X = torch.randn(60_000, dim, generator=g).cuda()
+    Q1 = torch.randn(300, dim, generator=g).cuda()
+    Q2 = torch.randn(41, dim, generator=g).cuda()      # the second call is smaller
+    dci = gpu.DCI(dim, M, L, B, T, seed=5, traversal=traversal)
+    dci.add(X)
+    lib = dci._lib
+    for Q in (Q1, Q2):
+        want = _call(dci, lib.dcih_query, Q, k, outer, B, T)
+        got = _call(dci, lib.dcih_query_noalloc, Q, k, outer, B, T)
+        assert torch.equal(got[0], want[0]), "ids differ"
+        assert torch.equal(got[1], want[1]), "distances differ"
+        assert torch.equal(got[2][:, 1], want[2][:, 1]) and torch.equal(got[2][:, 3], want[2][:, 3])
+        assert torch.all(got[0] >= 0)
+    # blind, also twice, second smaller
+    for Q in (Q1, Q2):
+        want = _call(dci, lib.dcih_query, Q, k, outer, B, T, blind=1)
+        got = _call(dci, lib.dcih_query_noalloc, Q, k, outer, B, T, blind=1)
+        assert torch.equal(got[0], want[0]) and torch.equal(got[1], want[1])
+    dci.free()
+
+
+def test_noalloc_rejects_what_does_not_fit(gpu):
+    from dciknn_cuda_amd import _capi
+    g = torch.Generator().manual_seed(22)
+    dim, B, T, k = 8, 64, 2, 50
+    X = torch.randn(40_000, dim, generator=g).cuda()
+    dci = gpu.DCI(dim, 2, 3, B, T, seed=5)
+    dci.add(X)
+    # 20000 queries * 64 partitions * 50 results * 8 bytes = 512 MB of result lists
+    Q = torch.randn(20_000, dim, generator=g).cuda()
+    ids = torch.empty((Q.shape[0], k), dtype=torch.int32, device="cuda")
+    dists = torch.empty((Q.shape[0], k), dtype=torch.float32, device="cuda")
+    rc = dci._lib.dcih_query_noalloc(dci._dci_inst, dim, Q.shape[0], Q.data_ptr(), k, 0, 30, 10 * k, B, T,
+                                     ids.data_ptr(), dists.data_ptr(), None, 0)
+    assert rc == -1
+    msg = dci._lib.dcih_last_error().decode()
+    assert "scratch" in msg and str(_capi.NOALLOC_SCRATCH_BYTES) in msg
+    # more results per query than the on-chip tables hold
+    rc = dci._lib.dcih_query_noalloc(dci._dci_inst, dim, 2, Q.data_ptr(), 9000, 0, 30, 90000, B, T,
+                                     ids.data_ptr(), dists.data_ptr(), None, 0)
+    assert rc == -4
+    # the allocating entry point still takes the large batch, and a small one still works here
+    _call(dci, dci._lib.dcih_query, Q, k, 30, B, T, counters=False)
+    a = _call(dci, dci._lib.dcih_query, Q[:64].contiguous(), k, 30, B, T)
+    b = _call(dci, dci._lib.dcih_query_noalloc, Q[:64].contiguous(), k, 30, B, T)
+    assert torch.equal(a[0], b[0]) and torch.equal(a[1], b[1])
+    dci.free()
