@@ -105,25 +105,41 @@ __global__ void segsort_tile_kernel(const float* __restrict__ keys, SegGeom g,
 // per-pass cost that does not depend on the slice (scan, barriers) grows with
 // the thread count, so the workgroup is the smallest of 64 / 128 / 256 / 512
 // threads that covers the slice with at most ~45 (512 threads: 63) items per
-// thread; a single wavefront needs no barrier at all.  Global traffic: keys
+// thread; a single wavefront needs no barrier at all.  The counters lie inside the
+// staging buffer (the items are in registers while they are in use), so a slice
+// takes 4 bytes of LDS per point and small slices share a CU.  Global traffic: keys
 // read once (all reads of a thread in flight together), sorted keys / ids /
 // inverse written once, all coalesced.
 constexpr int kRadixMax = 63 * 512;
 constexpr int kRadixMin = 512;        // up to this the bitonic tile kernel is faster
 constexpr int kRadixTile = 30 * 1024; // longest tile of a slice that needs merge passes
 
+// Waves per SIMD the register allocation leaves room for: as many workgroups as LDS lets
+// share a CU (one's passes then cover the other's loads, stores and barrier waits), but
+// never so many that the items no longer fit the registers.
+constexpr int radix_lds_bytes(int threads, int ipt) { return ((ipt > 8 ? ipt : 8) * threads + 64) * 4; }
+constexpr int radix_waves_per_simd(int threads, int ipt) {
+    const int by_lds = (160 * 1024 / radix_lds_bytes(threads, ipt)) * threads / 256;
+    const int by_regs = 512 / (2 * ipt + 86);
+    const int w = by_lds < by_regs ? by_lds : by_regs;
+    return w < 1 ? 1 : (w > 5 ? 5 : w);
+}
+
 template <int kRadixThreads, int IPT>
-// (256 threads with more than 45 items each: registers for two workgroups per CU)
-__global__ __launch_bounds__(kRadixThreads, (kRadixThreads == 256 && IPT > 45) ? 2 : 1) void segsort_radix_kernel(
+__global__ __launch_bounds__(kRadixThreads, radix_waves_per_simd(kRadixThreads, IPT)) void segsort_radix_kernel(
     const float* __restrict__ keys, SegGeom g, float* __restrict__ skeys,
     int32_t* __restrict__ sids, uint16_t* __restrict__ inv, uint16_t* __restrict__ lids,
     unsigned long long* __restrict__ packed) {
     extern __shared__ uint32_t rs[];
     uint32_t* stage = rs;                                         // IPT*1024 words
     uint16_t* stage16 = reinterpret_cast<uint16_t*>(rs);
-    uint16_t* cnt = reinterpret_cast<uint16_t*>(rs + IPT * kRadixThreads);   // [16][threads]
-    uint32_t* cnt32 = rs + IPT * kRadixThreads;
-    uint32_t* misc = rs + IPT * kRadixThreads + 8 * kRadixThreads;   // 64 words
+    // The digit counters share the staging buffer's room: between a pass's last read of the
+    // buffer and its next scatter the items live in registers.  A slice then needs 4 bytes
+    // of LDS per point, and two workgroups fit a CU up to 20 k points.
+    uint16_t* cnt = reinterpret_cast<uint16_t*>(rs);                 // [16][threads]
+    uint32_t* cnt32 = rs;
+    constexpr int kStageWords = IPT * kRadixThreads > 8 * kRadixThreads ? IPT * kRadixThreads : 8 * kRadixThreads;
+    uint32_t* misc = rs + kStageWords;                                // 64 words
 
     const int tid = threadIdx.x;
     const int lane = tid & 63, wave = tid >> 6;
@@ -184,17 +200,23 @@ __global__ __launch_bounds__(kRadixThreads, (kRadixThreads == 256 && IPT > 45) ?
             // A returning atomic on the word that holds the counter (two neighbouring
             // threads share a word): the LDS unit does the read-modify-write in issue
             // order, so the IPT updates of a thread need no round trip between them.
+            // (in batches, so that the returned values occupy few registers at a time)
             const uint32_t half = (uint32_t)(tid & 1) * 16u;
-            uint32_t old[IPT];
+            constexpr int kBatch = 13;
 #pragma unroll
-            for (int r = 0; r < IPT; r++) {
-                const uint32_t a = ((k[r] >> shift) & 15u) * kRadixThreads + tid;
-                old[r] = atomicAdd(&cnt32[a >> 1], 1u << half);
-                if ((r & 7) == 7) __builtin_amdgcn_sched_barrier(0);
+            for (int r0 = 0; r0 < IPT; r0 += kBatch) {
+                uint32_t old[kBatch];
+#pragma unroll
+                for (int r = r0; r < r0 + kBatch && r < IPT; r++) {
+                    const uint32_t a = ((k[r] >> shift) & 15u) * kRadixThreads + tid;
+                    old[r - r0] = atomicAdd(&cnt32[a >> 1], 1u << half);
+                }
+                __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+                for (int r = r0; r < r0 + kBatch && r < IPT; r++)
+                    rp[r] = (rp[r] & 0xffffu) | (((old[r - r0] >> half) & 0xffffu) << 16);
+                __builtin_amdgcn_sched_barrier(0);
             }
-#pragma unroll
-            for (int r = 0; r < IPT; r++)
-                rp[r] = (rp[r] & 0xffffu) | (((old[r] >> half) & 0xffffu) << 16);
         }
         __syncthreads();
         {   // exclusive scan of the 16*threads counters in memory order (digit-major)
@@ -230,6 +252,7 @@ __global__ __launch_bounds__(kRadixThreads, (kRadixThreads == 256 && IPT > 45) ?
             rp[r] += (uint32_t)cnt[a] << 16;                                      // would wait on each other
             if ((r & 7) == 7) __builtin_amdgcn_sched_barrier(0);
         }
+        __syncthreads();      // the scatter below overwrites the counters
         // (scheduling fences every 8 items keep the unrolled loops from computing all
         //  IPT addresses up front, which would spill registers)
 #pragma unroll
@@ -305,7 +328,7 @@ template <int NT, int IPT>
 static int launch_radix(const float* d_keys, const SegGeom& g, int num_indices, float* d_skeys,
                         int32_t* d_sids, uint16_t* d_inv, uint16_t* d_lids,
                         unsigned long long* d_packed, hipStream_t s) {
-    const size_t lds = (size_t)(IPT * NT + 8 * NT + 64) * sizeof(uint32_t);
+    const size_t lds = (size_t)radix_lds_bytes(NT, IPT);
     static DeviceOnce once;
     {
         const int rc = once.run([lds]() -> int {
