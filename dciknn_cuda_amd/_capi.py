@@ -12,7 +12,8 @@ LIB_PATH = os.path.join(_HERE, "libdci_hip.so")
 NUM_COUNTERS = 4
 CTR_VISITED, CTR_CANDIDATES, CTR_PROBES, CTR_STEPS = range(4)
 OPT_TRAVERSAL = 0
-TRAVERSAL_AUTO, TRAVERSAL_STEP, TRAVERSAL_BATCH = 0, 1, 2
+OPT_DENSE_MIN_PROMOTIONS = 1
+TRAVERSAL_AUTO, TRAVERSAL_STEP, TRAVERSAL_BATCH, TRAVERSAL_DENSE = 0, 1, 2, 3
 NOALLOC_SCRATCH_BYTES = 32 << 20
 NUM_TIMERS = 5
 T_PROJECT, T_SEGSORT, T_QPROJECT, T_TRAVERSE, T_MERGE = range(5)

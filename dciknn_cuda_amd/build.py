@@ -10,7 +10,7 @@ from concurrent.futures import ThreadPoolExecutor
 HERE = os.path.dirname(os.path.abspath(__file__))
 CSRC = os.path.join(HERE, "csrc")
 LIB = os.path.join(HERE, "libdci_hip.so")
-SOURCES = ["api.hip", "project.hip", "segsort.hip", "query.hip", "traverse_block.hip", "exhaustive.hip"]
+SOURCES = ["api.hip", "project.hip", "segsort.hip", "query.hip", "traverse_block.hip", "traverse_dense.hip", "exhaustive.hip"]
 HIPCC = os.environ.get("HIPCC", "/opt/rocm/bin/hipcc")
 FLAGS = [
     "-O3", "-std=c++17", "-fPIC", "--offload-arch=gfx950",

@@ -84,11 +84,12 @@ class DCI(object):
 
     def set_traversal(self, mode):
         """Pick the query kernel: "auto", "step" (one wavefront per partition,
-        one window per step) or "batch" (one workgroup per partition, whole index
-        ranges per epoch).  Both return the same neighbours."""
+        one window per step), "batch" (one workgroup per partition, whole index
+        ranges per epoch) or "dense" (one workgroup per partition, the promoting
+        step of every point at once).  All return the same neighbours."""
         self._require_handle()
         value = {"auto": _capi.TRAVERSAL_AUTO, "step": _capi.TRAVERSAL_STEP,
-                 "batch": _capi.TRAVERSAL_BATCH}[mode]
+                 "batch": _capi.TRAVERSAL_BATCH, "dense": _capi.TRAVERSAL_DENSE}[mode]
         _capi.check(self._lib.dcih_set_option(self._dci_inst, _capi.OPT_TRAVERSAL, value))
 
     def _require_handle(self):

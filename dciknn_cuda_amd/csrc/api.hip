@@ -131,6 +131,7 @@ struct dcih_index {
     float* d_stop_hint = nullptr;       // [3][block_size] epoch-size hints learnt from earlier queries
     int hint_k = 0, hint_outer = 0, hint_T = 0, hint_maxc = 0;   // query shape the hints belong to
     int traversal = 0;                  // DCIH_OPT_TRAVERSAL value
+    int dense_min_promos = 384;         // DCIH_OPT_DENSE_MIN_PROMOTIONS value
     unsigned long long* d_phase_ticks = nullptr;   // optional profile of the batch kernel
     // grow-only workspace: query scratch, and the unsorted keys during a build
     void* ws = nullptr;
@@ -519,6 +520,8 @@ static int query_impl(dcih_index* h, int dim, int num_queries, const float* d_qu
     a.skeys = h->d_skeys; a.sids = h->d_sids; a.inv = h->d_inv; a.lids = h->d_lids; a.data = h->d_data; a.query = d_query;
     a.mode = h->traversal; a.item_list = nullptr; a.item_count = nullptr; a.dense = nullptr;
     a.xcds = h->xcds; a.q_first = 0; a.q_count = num_queries;
+    a.dense_items = nullptr; a.dense_count = nullptr; a.dense_cap = 0;
+    a.dense_min_promos = h->dense_min_promos;
     a.phase_ticks = h->d_phase_ticks;
     // the hints describe where traversals of one query shape stop; forget them when it
     // changes (cleared by a kernel: a memset node is not safe in a captured graph)
@@ -597,7 +600,12 @@ static int query_impl(dcih_index* h, int dim, int num_queries, const float* d_qu
     const size_t part_bytes = align_up(query_part_bytes(a));
     const size_t gs_bytes = align_up(query_gscratch_bytes(a));
     const size_t redo_bytes = align_up((size_t)num_queries * block_size * sizeof(int32_t));
-    int rc = get_ws(qp_bytes + part_bytes + gs_bytes + redo_bytes + 256);
+    // per die one list of the items the batch kernel leaves to the dense kernel
+    a.dense_cap = (int64_t)num_queries * (block_size / h->xcds + 1) + 64;
+    const bool dense_lists = h->traversal == 0 && h->dense_min_promos > 0 && !blind &&
+                             dense_traversal_supported(a, nullptr) && block_traversal_supported(a, nullptr);
+    const size_t dense_bytes = dense_lists ? align_up((size_t)h->xcds * a.dense_cap * sizeof(int32_t)) : 0;
+    int rc = get_ws(qp_bytes + part_bytes + gs_bytes + redo_bytes + 256 + dense_bytes);
     if (rc) return rc;
     char* base = ws_base;
     float* d_qproj = (float*)base;
@@ -606,6 +614,8 @@ static int query_impl(dcih_index* h, int dim, int num_queries, const float* d_qu
     a.gscratch = gs_bytes ? (uint32_t*)(base + qp_bytes + part_bytes) : nullptr;
     a.redo_items = (int32_t*)(base + qp_bytes + part_bytes + gs_bytes);
     a.redo_count = (uint32_t*)(base + qp_bytes + part_bytes + gs_bytes + redo_bytes);
+    a.dense_count = a.redo_count + 1;         // one length per die, cleared together with redo_count
+    a.dense_items = dense_lists ? (int32_t*)(base + qp_bytes + part_bytes + gs_bytes + redo_bytes + 256) : nullptr;
 
     mark(h, DCIH_T_QPROJECT, 0, s);
     rc = project(h->d_dirs, I, d_query, num_queries, dim, d_qproj, num_queries, s);
@@ -657,8 +667,12 @@ int64_t dcih_debug_launch_map(int xcds, int block_size, int num_queries, int64_t
 
 int dcih_set_option(dcih_index* h, int option, int value) {
     if (!h) return fail(DCIH_EINVAL, "dcih_set_option: null handle");
-    if (option == DCIH_OPT_TRAVERSAL && value >= 0 && value <= 2) {
+    if (option == DCIH_OPT_TRAVERSAL && value >= 0 && value <= 3) {
         h->traversal = value;
+        return DCIH_OK;
+    }
+    if (option == DCIH_OPT_DENSE_MIN_PROMOTIONS && value >= 0) {
+        h->dense_min_promos = value;
         return DCIH_OK;
     }
     return fail(DCIH_EINVAL, "dcih_set_option: unknown option or value");

@@ -51,7 +51,12 @@ struct QueryArgs {
     const uint32_t* item_count;  // ... of this length
     float* stop_hint;        // null, or [3][B] per partition: running averages of the stop step and of the promotions at the stop, stops seen
     unsigned long long* phase_ticks;  // null, or 16 accumulators for the batch kernel's phases
-    int mode;                // 0 = pick, 1 = step-by-step kernel, 2 = batch kernel
+    int mode;                // 0 = pick, 1 = step-by-step kernel, 2 = batch kernel, 3 = dense kernel
+    // hand-over from the batch kernel to the dense kernel: one list of items per die
+    int32_t* dense_items;    // null, or [xcds][dense_cap]
+    uint32_t* dense_count;   // [xcds]
+    int64_t dense_cap;
+    int dense_min_promos;    // promotions per (query, partition) from which the dense kernel is the cheaper one
     int xcds;                // accelerator dies of the device (each has an L2 of its own)
     int q_first, q_count;    // batch kernel: the queries one launch covers
     int32_t* out_ids;        // [nq][k]
@@ -108,6 +113,11 @@ size_t query_gscratch_bytes(const QueryArgs& a);
 // tables, and the launch itself.
 bool block_traversal_supported(const QueryArgs& a, size_t* lds_bytes);
 int query_block(const QueryArgs& a, hipStream_t s);
+// Dense traversal (traverse_dense.hip): every point's promoting step at once.  Works
+// through the lists the batch kernel filled (a.dense_items) or, with a.mode == 3,
+// through all items.
+bool dense_traversal_supported(const QueryArgs& a, size_t* lds_bytes);
+int query_dense_items(const QueryArgs& a, hipStream_t s);
 
 // Full ranking (exhaustive.hip) for num_neighbours above the points per partition,
 // where the traversal provably visits everything: queries are processed `chunk` at

@@ -306,10 +306,11 @@ __global__ __launch_bounds__(kMergeThreads) void merge_topk_kernel(QueryArgs a, 
     }
 }
 
-__global__ void zero_u64_kernel(unsigned long long* p, int64_t n, uint32_t* also) {
+// Clears n 64-bit words at p and also_n 32-bit words at `also` (either may be null / 0).
+__global__ void zero_u64_kernel(unsigned long long* p, int64_t n, uint32_t* also, int also_n) {
     const int64_t stride = (int64_t)gridDim.x * blockDim.x;
     for (int64_t e = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; e < n; e += stride) p[e] = 0;
-    if (also && blockIdx.x == 0 && threadIdx.x == 0) *also = 0;
+    if (also && blockIdx.x == 0 && (int)threadIdx.x < also_n) also[threadIdx.x] = 0;
 }
 
 int merge_cap(int k) {
@@ -337,7 +338,7 @@ static int allow_full_lds() {
 int zero_words64(void* d_p, int64_t n, hipStream_t s) {
     if (n <= 0) return 0;
     hipLaunchKernelGGL(zero_u64_kernel, dim3((unsigned)max((int64_t)1, min((int64_t)1024, (n + 255) / 256))),
-                       dim3(256), 0, s, (unsigned long long*)d_p, n, (uint32_t*)nullptr);
+                       dim3(256), 0, s, (unsigned long long*)d_p, n, (uint32_t*)nullptr, 0);
     DCIH_HIP(hipGetLastError());
     return 0;
 }
@@ -372,25 +373,39 @@ int query(const QueryArgs& a_in, hipStream_t s, hipEvent_t* ev) {
     if (y.lds_bytes > (size_t)kMaxLds)
         return fail(-4, "query: dim / num_indices / num_neighbours too large for LDS state");
     const bool can_block = block_traversal_supported(a, nullptr);
+    const bool can_dense = dense_traversal_supported(a, nullptr);
     if (a.mode == 2 && !can_block)
         return fail(-4, "query: this shape does not fit the batch traversal kernel");
-    const bool use_block = a.mode != 1 && can_block;
+    if (a.mode == 3 && !can_dense)
+        return fail(-4, "query: this shape does not fit the dense traversal kernel");
+    const bool use_block = a.mode != 1 && a.mode != 3 && can_block;
+    // the batch kernel hands items that need many promotions to the dense kernel
+    if (!(use_block && a.mode == 0 && can_dense && a.dense_items && a.dense_min_promos > 0)) {
+        if (a.mode != 3) a.dense_items = nullptr;
+    }
     {
         const int rc = allow_full_lds();
         if (rc) return rc;
     }
-    {   // zero the counters and the redo count with a kernel (safe under graph capture)
+    {   // zero the counters and the list lengths with a kernel (safe under graph capture);
+        // the dense lists' lengths follow the hand-over list's
         const int64_t cells = a.counters ? (int64_t)a.nq * 4 : 0;
         hipLaunchKernelGGL(zero_u64_kernel, dim3((unsigned)max((int64_t)1, min((int64_t)1024, (cells + 255) / 256))),
-                           dim3(256), 0, s, a.counters, cells, a.redo_count);
+                           dim3(256), 0, s, a.counters, cells, a.redo_count, 1 + a.xcds);
     }
     if (ev) (void)hipEventRecord(ev[0], s);
     a.item_list = nullptr;
     a.item_count = nullptr;
-    if (use_block) {
-        const int rc = query_block(a, s);
-        if (rc) return rc;
-        // whatever the batch kernel handed back goes through the step-by-step kernel
+    if (use_block || a.mode == 3) {
+        if (use_block) {
+            const int rc = query_block(a, s);
+            if (rc) return rc;
+        }
+        if (a.mode == 3 || a.dense_items) {
+            const int rc = query_dense_items(a, s);
+            if (rc) return rc;
+        }
+        // whatever those kernels handed back goes through the step-by-step kernel
         a.item_list = a.redo_items;
         a.item_count = a.redo_count;
         const int64_t grid = min((int64_t)a.nq * a.B, (int64_t)1024);
@@ -449,7 +464,7 @@ int query_dense(const QueryArgs& a_in, const float* d_dirs, void* ws, int chunk,
             return fail(-4, "query: dim / num_indices too large for LDS state");
         const int64_t cells = a.counters ? (int64_t)a.nq * 4 : 0;
         hipLaunchKernelGGL(zero_u64_kernel, dim3((unsigned)max((int64_t)1, min((int64_t)1024, (cells + 255) / 256))),
-                           dim3(256), 0, s, a.counters, cells, (uint32_t*)nullptr);
+                           dim3(256), 0, s, a.counters, cells, (uint32_t*)nullptr, 0);
         const int64_t grid = traverse_grid(a, y);
         if (y.lds_counters) {
             hipLaunchKernelGGL(traverse_kernel<true>, dim3((unsigned)grid), dim3(kWave), y.lds_bytes, s, a, y);

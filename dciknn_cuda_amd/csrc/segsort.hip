@@ -13,6 +13,7 @@
 // pass doubling the run length, the last one writing the final arrays.
 #include "common.h"
 #include "kernels.h"
+#include "radix_core.h"
 
 namespace dcih {
 
@@ -105,41 +106,25 @@ __global__ void segsort_tile_kernel(const float* __restrict__ keys, SegGeom g,
 // per-pass cost that does not depend on the slice (scan, barriers) grows with
 // the thread count, so the workgroup is the smallest of 64 / 128 / 256 / 512
 // threads that covers the slice with at most ~45 (512 threads: 63) items per
-// thread; a single wavefront needs no barrier at all.  The counters lie inside the
-// staging buffer (the items are in registers while they are in use), so a slice
-// takes 4 bytes of LDS per point and small slices share a CU.  Global traffic: keys
+// thread; a single wavefront needs no barrier at all.  Global traffic: keys
 // read once (all reads of a thread in flight together), sorted keys / ids /
 // inverse written once, all coalesced.
 constexpr int kRadixMax = 63 * 512;
 constexpr int kRadixMin = 512;        // up to this the bitonic tile kernel is faster
 constexpr int kRadixTile = 30 * 1024; // longest tile of a slice that needs merge passes
 
-// Waves per SIMD the register allocation leaves room for: as many workgroups as LDS lets
-// share a CU (one's passes then cover the other's loads, stores and barrier waits), but
-// never so many that the items no longer fit the registers.
-constexpr int radix_lds_bytes(int threads, int ipt) { return ((ipt > 8 ? ipt : 8) * threads + 64) * 4; }
-constexpr int radix_waves_per_simd(int threads, int ipt) {
-    const int by_lds = (160 * 1024 / radix_lds_bytes(threads, ipt)) * threads / 256;
-    const int by_regs = 512 / (2 * ipt + 86);
-    const int w = by_lds < by_regs ? by_lds : by_regs;
-    return w < 1 ? 1 : (w > 5 ? 5 : w);
-}
+constexpr int radix_lds_bytes(int threads, int ipt) { return (ipt * threads + 8 * threads + 64) * 4; }
 
 template <int kRadixThreads, int IPT>
-__global__ __launch_bounds__(kRadixThreads, radix_waves_per_simd(kRadixThreads, IPT)) void segsort_radix_kernel(
+__global__ __launch_bounds__(kRadixThreads, (kRadixThreads == 256 && IPT > 45) ? 2 : 1) void segsort_radix_kernel(
     const float* __restrict__ keys, SegGeom g, float* __restrict__ skeys,
     int32_t* __restrict__ sids, uint16_t* __restrict__ inv, uint16_t* __restrict__ lids,
     unsigned long long* __restrict__ packed) {
     extern __shared__ uint32_t rs[];
     uint32_t* stage = rs;                                         // IPT*1024 words
     uint16_t* stage16 = reinterpret_cast<uint16_t*>(rs);
-    // The digit counters share the staging buffer's room: between a pass's last read of the
-    // buffer and its next scatter the items live in registers.  A slice then needs 4 bytes
-    // of LDS per point, and two workgroups fit a CU up to 20 k points.
-    uint16_t* cnt = reinterpret_cast<uint16_t*>(rs);                 // [16][threads]
-    uint32_t* cnt32 = rs;
-    constexpr int kStageWords = IPT * kRadixThreads > 8 * kRadixThreads ? IPT * kRadixThreads : 8 * kRadixThreads;
-    uint32_t* misc = rs + kStageWords;                                // 64 words
+    uint32_t* cnt32 = rs + IPT * kRadixThreads;                      // digit counters, [16][threads] 16-bit
+    uint32_t* misc = rs + IPT * kRadixThreads + 8 * kRadixThreads;   // 64 words
 
     const int tid = threadIdx.x;
     const int lane = tid & 63, wave = tid >> 6;
@@ -190,95 +175,7 @@ __global__ __launch_bounds__(kRadixThreads, radix_waves_per_simd(kRadixThreads, 
     __syncthreads();
     const uint32_t varying = misc[32] ^ misc[33];
 
-    for (int shift = 0; shift < 32; shift += 4) {
-        if (((varying >> shift) & 15u) == 0u) continue;          // same nibble everywhere
-        __syncthreads();
-        {   // count digits in thread-private LDS counters (no atomics, order-preserving)
-#pragma unroll
-            for (int w = 0; w < 8; w++) cnt32[tid + w * kRadixThreads] = 0;
-            __syncthreads();
-            // A returning atomic on the word that holds the counter (two neighbouring
-            // threads share a word): the LDS unit does the read-modify-write in issue
-            // order, so the IPT updates of a thread need no round trip between them.
-            // (in batches, so that the returned values occupy few registers at a time)
-            const uint32_t half = (uint32_t)(tid & 1) * 16u;
-            constexpr int kBatch = 13;
-#pragma unroll
-            for (int r0 = 0; r0 < IPT; r0 += kBatch) {
-                uint32_t old[kBatch];
-#pragma unroll
-                for (int r = r0; r < r0 + kBatch && r < IPT; r++) {
-                    const uint32_t a = ((k[r] >> shift) & 15u) * kRadixThreads + tid;
-                    old[r - r0] = atomicAdd(&cnt32[a >> 1], 1u << half);
-                }
-                __builtin_amdgcn_sched_barrier(0);
-#pragma unroll
-                for (int r = r0; r < r0 + kBatch && r < IPT; r++)
-                    rp[r] = (rp[r] & 0xffffu) | (((old[r - r0] >> half) & 0xffffu) << 16);
-                __builtin_amdgcn_sched_barrier(0);
-            }
-        }
-        __syncthreads();
-        {   // exclusive scan of the 16*threads counters in memory order (digit-major)
-            uint32_t v[8];
-            uint32_t sum = 0;
-#pragma unroll
-            for (int w = 0; w < 8; w++) { v[w] = cnt32[tid * 8 + w]; sum += (v[w] & 0xffffu) + (v[w] >> 16); }
-            uint32_t incl = sum;
-#pragma unroll
-            for (int o = 1; o < 64; o <<= 1) {
-                const uint32_t t = (uint32_t)__shfl_up((int)incl, o, 64);
-                if (lane >= o) incl += t;
-            }
-            if (lane == 63) misc[wave] = incl;
-            __syncthreads();
-            uint32_t run = incl - sum;
-            for (int w2 = 0; w2 < wave; w2++) run += misc[w2];
-#pragma unroll
-            for (int w = 0; w < 8; w++) {
-                const uint32_t lo = v[w] & 0xffffu, hi = v[w] >> 16;
-                cnt32[tid * 8 + w] = run | ((run + lo) << 16);
-                run += lo + hi;
-            }
-        }
-        __syncthreads();
-        // an opaque copy of the shift keeps the compiler from holding all IPT counter
-        // addresses of the counting loop alive across the scan
-        int shift2 = shift;
-        asm volatile("" : "+s"(shift2));
-#pragma unroll
-        for (int r = 0; r < IPT; r++) {      // all counter reads first, then all stores:
-            const uint32_t a = ((k[r] >> shift2) & 15u) * kRadixThreads + tid;   // interleaved they
-            rp[r] += (uint32_t)cnt[a] << 16;                                      // would wait on each other
-            if ((r & 7) == 7) __builtin_amdgcn_sched_barrier(0);
-        }
-        __syncthreads();      // the scatter below overwrites the counters
-        // (scheduling fences every 8 items keep the unrolled loops from computing all
-        //  IPT addresses up front, which would spill registers)
-#pragma unroll
-        for (int r = 0; r < IPT; r++) {
-            stage[rp[r] >> 16] = k[r];
-            if ((r & 7) == 7) __builtin_amdgcn_sched_barrier(0);
-        }
-        __syncthreads();
-#pragma unroll
-        for (int r = 0; r < IPT; r++) {
-            k[r] = stage[tid * IPT + r];
-            if ((r & 7) == 7) __builtin_amdgcn_sched_barrier(0);
-        }
-        __syncthreads();
-#pragma unroll
-        for (int r = 0; r < IPT; r++) {      // ids move as whole words: 16-bit blocked reads would
-            stage[rp[r] >> 16] = rp[r] & 0xffffu;                // collide on LDS banks
-            if ((r & 7) == 7) __builtin_amdgcn_sched_barrier(0);
-        }
-        __syncthreads();
-#pragma unroll
-        for (int r = 0; r < IPT; r++) {
-            rp[r] = stage[tid * IPT + r];
-            if ((r & 7) == 7) __builtin_amdgcn_sched_barrier(0);
-        }
-    }
+    lds_radix_passes<kRadixThreads, IPT>(k, rp, stage, cnt32, misc, varying);
 
     if (packed) {      // (same on every thread) keys, then ids, through LDS into coalesced order
         __syncthreads();

@@ -1,0 +1,498 @@
+// Dense traversal: one workgroup per (query, partition) computes, for EVERY point
+// of the partition, the outer step at which the loop of
+// dci_query_single_point_by_block (src/dci_cuda_kernel.cu:401-626) would promote
+// it, and from those steps the stop step, the candidates and their k best.
+//
+// It is the kernel for traversals that visit a large part of the index before
+// they stop (hundreds or thousands of promotions per partition): there the batch
+// kernel's cost per promotion (a rank by 2L binary searches, a replay) dominates,
+// while the work here does not depend on where the loop stops.  Facts used, the
+// same as in the batch kernel: a composite index consumes its windows in
+// ascending (priority, simple index, order within the simple index), window
+// number r at outer step r; a point is promoted under a composite at the step of
+// the last of the L windows that hold it and is a candidate at its earliest
+// (step, composite); the loop stops at the first step t with c0(t) >= k and
+// (t + 1 >= outer * L or c0(t) >= max_candidates), c0 counting candidates whose
+// promoting window held them in lane 0 (:598-607).
+//
+// Per composite index: the priorities |key[clamped window start] - q| (:572-590)
+// of all its windows are laid out by (simple index, order within it) and sorted
+// stably in LDS, which gives every window its step; every point then looks up the
+// steps of its L windows (positions from the inverse permutation) and keeps the
+// largest.  A histogram of the steps of lane-0 candidates yields the stop step;
+// points promoted up to it get their exact distances (rows read by whole
+// wavefronts) and go through a k-best filter.  Shapes that do not fit the tables
+// are left to the other kernels through the same hand-over list.
+#include "common.h"
+#include "kernels.h"
+#include "radix_core.h"
+#include "traverse_common.h"
+
+namespace dcih {
+
+namespace {
+
+constexpr int kDT = 256;                 // threads per workgroup
+constexpr int kDWaves = kDT / kWave;
+constexpr uint32_t kNever = 0xffffu;     // step field of a point that is never promoted
+
+enum DMisc {   // 32-bit scalars shared by the workgroup
+    dWin = 0, dFail, dArmed, dMaxc, dCand, dProbes, dMore, dOr, dAnd, dMaxW, dWavePend0,
+    dMiscWords = 16
+};
+
+struct DenseLayout {
+    int ipt;          // windows per thread the sort holds (cap = 256 * ipt per composite)
+    int off_idx;      // per simple index: p, qp, left start, right start   (4 * I words)
+    int off_seg;      // per composite: 2L + 1 segment starts, 2L stream numbers
+    int off_q;        // query row
+    int off_time;     // uint16 per point: step << 1 | lane-0 flag
+    int off_sort;     // k best + pending candidates, 64-bit words
+    int off_stage;    // radix staging; later the rank table, then the step histogram
+    int off_misc;
+    int sort_cap, quota;
+    size_t lds_bytes;
+};
+
+int dense_ipt_for(int64_t windows) {
+    for (int ipt : {9, 17, 25, 33})
+        if (windows <= (int64_t)kDT * ipt) return ipt;
+    return 0;
+}
+
+// Upper bound of the windows of one composite index: per simple index at most
+// ceil((p+1)/T) + floor((n+T-3-p)/T) + 1 <= n/T + 3.
+int64_t dense_max_windows(const QueryArgs& a) { return (int64_t)a.L * (a.ppb / a.T + 3); }
+
+DenseLayout make_dense_layout(const QueryArgs& a) {
+    DenseLayout y;
+    const int I = a.M * a.L;
+    y.ipt = dense_ipt_for(dense_max_windows(a));
+    int o = dMiscWords * 4 + 64 * 4;      // scalars, then scratch of the block scans
+    y.off_misc = 0;
+    y.off_idx = o;      o += 4 * I * 4;
+    y.off_seg = o;      o += (4 * a.L + 2) * 4;
+    y.off_q = o;        o += ((a.dim + 3) & ~3) * 4;
+    y.off_time = o;     o += (int)(((a.ppb + 1) & ~(int64_t)1) * 2);
+    o = (o + 15) & ~15;
+    // k best plus room for candidates that beat the current k-th: four wavefronts fill
+    // a quota each between two merges
+    y.sort_cap = 64;
+    while (y.sort_cap < a.kcap + 4 * 8) y.sort_cap <<= 1;
+    y.quota = (y.sort_cap - a.kcap) / kDWaves;
+    y.off_sort = o;     o += y.sort_cap * 8;
+    y.off_stage = o;    o += (y.ipt + 8) * kDT * 4;      // staging words, then the digit counters
+    y.lds_bytes = (size_t)o;
+    return y;
+}
+
+template <int IPT>
+__global__ __launch_bounds__(kDT, 2) void traverse_dense_kernel(QueryArgs a, DenseLayout y) {
+    extern __shared__ __align__(16) unsigned char smem[];
+    uint32_t* misc = reinterpret_cast<uint32_t*>(smem);
+    uint32_t* scan_tmp = misc + dMiscWords;                           // 64 words
+    int* s_p = reinterpret_cast<int*>(smem + y.off_idx);
+    float* s_qp = reinterpret_cast<float*>(s_p + a.M * a.L);
+    int* s_startL = reinterpret_cast<int*>(s_qp + a.M * a.L);         // layout index of a stream's window 0
+    int* s_startR = s_startL + a.M * a.L;
+    int* s_seg = reinterpret_cast<int*>(smem + y.off_seg);            // 2L + 1 segment starts (layout order)
+    int* s_segstream = s_seg + 2 * a.L + 1;                           // stream (2h + side) of a segment
+    float* s_q = reinterpret_cast<float*>(smem + y.off_q);
+    uint16_t* s_time = reinterpret_cast<uint16_t*>(smem + y.off_time);
+    unsigned long long* sortbuf = reinterpret_cast<unsigned long long*>(smem + y.off_sort);
+    uint32_t* stage = reinterpret_cast<uint32_t*>(smem + y.off_stage);
+    uint16_t* rank16 = reinterpret_cast<uint16_t*>(stage);
+
+    const int tid = threadIdx.x;
+    const int lane = tid & (kWave - 1);
+    const int wave = tid / kWave;
+    const int I = a.M * a.L;
+    const int T = a.T;
+    const uint32_t T_magic = a.T_magic;
+    auto div_T = [&](int d) { return T > 1 ? (int)__umulhi((uint32_t)d, T_magic) : d; };
+    const int X = a.xcds;
+    const int xcd = (int)(blockIdx.x % X);
+    const int64_t g0 = blockIdx.x / X, G = gridDim.x / X;
+    const bool listed = a.dense_items != nullptr && a.mode != 3;
+    const int64_t my_count = listed ? (int64_t)a.dense_count[xcd]
+                                    : block_items(X, a.B, a.q_count) / X;
+
+    for (int64_t slot = g0; slot < my_count; slot += G) {
+        int b, qi;
+        if (listed) {
+            const int64_t item = a.dense_items[(int64_t)xcd * a.dense_cap + slot];
+            b = (int)(item % a.B);
+            qi = (int)(item / a.B);
+        } else {
+            if (!block_item(slot * X + xcd, X, a.B, a.q_count, b, qi)) continue;
+            qi += a.q_first;
+        }
+        const int64_t item = (int64_t)qi * a.B + b;
+        const int64_t off = (int64_t)b * a.ppb;
+        const int n = (int)min(a.N - off, a.ppb);
+        unsigned long long* part_out = a.part + item * a.kcap;
+        __syncthreads();                         // the previous item's tables are done with
+        if (n <= 0) {
+            for (int j = tid; j < a.kcap; j += kDT) part_out[j] = ~0ull;
+            continue;
+        }
+
+        // ---- set-up: query row, positioning searches (:279-297) -------------------
+        if (tid < dMiscWords) misc[tid] = 0;
+        for (int j = tid; j < a.dim; j += kDT) s_q[j] = a.query[(int64_t)qi * a.dim + j];
+        for (int pt = tid; pt < n; pt += kDT) s_time[pt] = (uint16_t)((kNever << 1) & 0xffffu);
+        uint32_t probes = 0;
+        {
+            const int per_wave = (I + kDWaves - 1) / kDWaves;
+            const int lg = min(3, floor_log2(kWave / per_wave > 0 ? kWave / per_wave : 1)), Gq = 1 << lg;
+            const int slots = kWave >> lg;
+            for (int i0 = 0; i0 < I; i0 += slots * kDWaves) {
+                const int sl = lane >> lg, i = i0 + wave * slots + sl;
+                const bool active = i < I;
+                const float* key = a.skeys + (int64_t)(active ? i : 0) * a.N + off;
+                const float qp = active ? a.qproj[(int64_t)i * a.nq + qi] : 0.f;
+                const int lo = group_partition_point(0, n, active, lg, sl * Gq, lane - sl * Gq,
+                                                     [&](int j) { return key[j] < qp; }, probes);
+                if (active && lane == sl * Gq) { s_p[i] = lo - 1; s_qp[i] = qp; }
+            }
+        }
+        __syncthreads();
+
+        unsigned long long maxw = 0;             // most windows any composite has
+        for (int m = 0; m < a.M; m++) {
+            // ---- layout of the composite's windows: per simple index its left stream, then
+            // its right one; where the query lies above every key the single (ghost) right
+            // window comes first, as dci_next_closest_proj orders it (:264-265)
+            if (tid == 0) {
+                int at = 0;
+                for (int h = 0; h < a.L; h++) {
+                    const int i = m * a.L + h, p = s_p[i];
+                    const int nl = stream_windows(n, T, p, 0), nr = stream_windows(n, T, p, 1);
+                    const bool corner = p == n - 1 && T >= 2;
+                    if (corner) {
+                        s_seg[2 * h] = at; s_segstream[2 * h] = 2 * h + 1; s_startR[i] = at; at += nr;
+                        s_seg[2 * h + 1] = at; s_segstream[2 * h + 1] = 2 * h; s_startL[i] = at; at += nl;
+                    } else {
+                        s_seg[2 * h] = at; s_segstream[2 * h] = 2 * h; s_startL[i] = at; at += nl;
+                        s_seg[2 * h + 1] = at; s_segstream[2 * h + 1] = 2 * h + 1; s_startR[i] = at; at += nr;
+                    }
+                }
+                s_seg[2 * a.L] = at;
+                misc[dWin] = (uint32_t)at;
+                if (at > kDT * IPT || at >= 0x7fff) misc[dFail] = 1;
+                misc[dOr] = 0; misc[dAnd] = 0xffffffffu;
+            }
+            __syncthreads();
+            if (misc[dFail]) break;
+            const int W = (int)misc[dWin];
+            maxw = max(maxw, (unsigned long long)W);
+
+            // ---- priorities of the windows, blocked: thread t holds layout indices t*IPT.. ----
+            uint32_t k[IPT], rp[IPT];
+            {
+                int seg = 0;
+                const int first = tid * IPT;
+                while (seg < 2 * a.L - 1 && s_seg[seg + 1] <= first) seg++;
+                int seg_end = s_seg[seg + 1];
+                int sidx = s_segstream[seg];
+                int seg_at = s_seg[seg];
+                // (offsets from the composite's first slice; all reads are issued before any is used)
+                const float* kbase = a.skeys + (int64_t)m * a.L * a.N + off;
+                uint32_t koff[IPT];
+                float qv[IPT];
+#pragma unroll
+                for (int r = 0; r < IPT; r++) {
+                    const int idx = first + r;
+                    while (idx >= seg_end && seg < 2 * a.L - 1) {
+                        seg++;
+                        seg_end = s_seg[seg + 1]; sidx = s_segstream[seg]; seg_at = s_seg[seg];
+                    }
+                    const int h = sidx >> 1, p = s_p[m * a.L + h], j = idx - seg_at;
+                    const int pos = (sidx & 1) ? min(p + 1 + j * T, n - 1) : max(p - T + 1 - j * T, 0);
+                    koff[r] = (uint32_t)h * (uint32_t)a.N + (uint32_t)(idx < W ? pos : 0);
+                    qv[r] = s_qp[m * a.L + h];
+                }
+                float kv[IPT];
+#pragma unroll
+                for (int r = 0; r < IPT; r++) kv[r] = kbase[koff[r]];
+                uint32_t vor = 0, vand = 0xffffffffu;
+#pragma unroll
+                for (int r = 0; r < IPT; r++) {
+                    const int idx = first + r;
+                    const uint32_t bits = __builtin_bit_cast(uint32_t, fabsf(kv[r] - qv[r]));
+                    k[r] = idx < W ? bits : 0xffffffffu;      // pads sort last and stay last
+                    rp[r] = (uint32_t)idx;
+                    vor |= idx < W ? bits : 0u;
+                    vand &= idx < W ? bits : 0xffffffffu;
+                }
+                probes += IPT;
+                for (int o = 32; o > 0; o >>= 1) {
+                    vor |= (uint32_t)__shfl_xor((int)vor, o, kWave);
+                    vand &= (uint32_t)__shfl_xor((int)vand, o, kWave);
+                }
+                if (lane == 0) { atomicOr(&misc[dOr], vor); atomicAnd(&misc[dAnd], vand); }
+            }
+            __syncthreads();
+            // (the pads need no pass of their own: they start behind every window, every
+            //  digit of theirs is the largest, and the passes are stable)
+            const uint32_t varying = misc[dOr] ^ misc[dAnd];
+            lds_radix_passes<kDT, IPT>(k, rp, stage, stage + IPT * kDT, scan_tmp, varying);
+            __syncthreads();
+            // the step of every window: its place in the sorted order
+#pragma unroll
+            for (int r = 0; r < IPT; r++) {
+                const uint32_t idx = rp[r] & 0xffffu;
+                if (idx < (uint32_t)W) rank16[idx] = (uint16_t)(tid * IPT + r);
+            }
+            __syncthreads();
+
+            // ---- every point: the latest of the steps of its L windows ------------------
+            // (sixteen points per thread at a time, so that as many reads of the inverse
+            //  permutation are in flight)
+            constexpr int kP = 16;
+            const uint16_t* invm = a.inv + (int64_t)m * a.L * a.N + off;
+            for (int c0 = 0; c0 < n; c0 += kDT * kP) {
+                int tmax[kP];
+                uint32_t l0mask = 0;
+#pragma unroll
+                for (int u = 0; u < kP; u++) tmax[u] = -1;
+                for (int h = 0; h < a.L; h++) {
+                    const int i = m * a.L + h;
+                    const int p = s_p[i], sl = s_startL[i], sr = s_startR[i];
+                    const uint16_t* invh = invm + (int64_t)h * a.N;
+                    int posv[kP];
+#pragma unroll
+                    for (int u = 0; u < kP; u++) posv[u] = (int)invh[min(c0 + u * kDT + tid, n - 1)];
+#pragma unroll
+                    for (int u = 0; u < kP; u++) {
+                        const int pos = posv[u];
+                        int idx, t;
+                        if (pos > p) {
+                            const int d = pos - (p + 1), j = div_T(d);
+                            t = d - j * T; idx = sr + j;
+                        } else {
+                            const int d = p - pos, j = div_T(d);
+                            t = pos - (p - T + 1 - j * T); idx = sl + j;
+                        }
+                        const int r = (int)rank16[idx];
+                        if (r > tmax[u]) {
+                            tmax[u] = r;
+                            l0mask = (l0mask & ~(1u << u)) | ((t == 0 ? 1u : 0u) << u);
+                        }
+                    }
+                }
+#pragma unroll
+                for (int u = 0; u < kP; u++) {
+                    const int pt = c0 + u * kDT + tid;
+                    if (pt < n) {
+                        const uint32_t old = s_time[pt];      // ties: the earlier composite stays
+                        if ((uint32_t)tmax[u] < (old >> 1)) s_time[pt] = (uint16_t)((tmax[u] << 1) | ((l0mask >> u) & 1u));
+                    }
+                }
+            }
+            __syncthreads();
+        }
+        if (misc[dFail]) {      // does not fit the tables: the step-by-step kernel takes the item
+            if (tid == 0) {
+                const uint32_t s2 = atomicAdd(a.redo_count, 1u);
+                a.redo_items[s2] = (int32_t)item;
+            }
+            continue;
+        }
+
+        // ---- stop step from the histogram of the steps of lane-0 candidates -----------
+        const int HW = ((int)maxw + 2) / 2;                 // 32-bit words of the histogram (two steps each)
+        for (int w = tid; w < HW; w += kDT) stage[w] = 0;
+        if (tid == 0) { misc[dArmed] = 0xffffffffu; misc[dMaxc] = 0xffffffffu; }
+        __syncthreads();
+        for (int pt = tid; pt < n; pt += kDT) {
+            const uint32_t v = s_time[pt];
+            if ((v & 1u) && (v >> 1) != (kNever & 0x7fffu)) atomicAdd(&stage[v >> 2], 1u << (((v >> 1) & 1u) * 16));
+        }
+        __syncthreads();
+        {
+            const int per = (HW + kDT - 1) / kDT;           // words per thread, contiguous
+            const int w0 = tid * per, w1 = min(HW, w0 + per);
+            uint32_t sum = 0;
+            for (int w = w0; w < w1; w++) { const uint32_t v = stage[w]; sum += (v & 0xffffu) + (v >> 16); }
+            uint32_t incl = sum;
+#pragma unroll
+            for (int o = 1; o < kWave; o <<= 1) {
+                const uint32_t t2 = (uint32_t)__shfl_up((int)incl, o, kWave);
+                if (lane >= o) incl += t2;
+            }
+            if (lane == kWave - 1) scan_tmp[wave] = incl;
+            __syncthreads();
+            uint32_t run = incl - sum;
+            for (int w2 = 0; w2 < wave; w2++) run += scan_tmp[w2];
+            const uint32_t need_k = (uint32_t)a.k_stop;
+            const uint32_t need_c = (uint32_t)min((int64_t)0x7fffffff, max((int64_t)1, a.max_cand));
+            for (int w = w0; w < w1; w++) {
+                const uint32_t v = stage[w];
+                const uint32_t c_lo = run + (v & 0xffffu), c_hi = c_lo + (v >> 16);
+                if (run < need_k && c_lo >= need_k) atomicMin(&misc[dArmed], (uint32_t)(2 * w));
+                else if (c_lo < need_k && c_hi >= need_k) atomicMin(&misc[dArmed], (uint32_t)(2 * w + 1));
+                if (run < need_c && c_lo >= need_c) atomicMin(&misc[dMaxc], (uint32_t)(2 * w));
+                else if (c_lo < need_c && c_hi >= need_c) atomicMin(&misc[dMaxc], (uint32_t)(2 * w + 1));
+                run = c_hi;
+            }
+        }
+        __syncthreads();
+        const uint32_t t_armed = misc[dArmed], t_maxc = misc[dMaxc];
+        const bool stop = t_armed != 0xffffffffu;
+        unsigned long long t_stop = ~0ull;                  // candidates: promoted at a step <= t_stop
+        if (stop) {
+            const unsigned long long last_needed = a.stop_at > 0 ? (unsigned long long)(a.stop_at - 1) : 0ull;
+            const unsigned long long by_count = t_maxc != 0xffffffffu ? (unsigned long long)t_maxc : ~0ull;
+            t_stop = max((unsigned long long)t_armed, min(last_needed, by_count));
+        }
+        const uint32_t t_lim = (uint32_t)min(t_stop, (unsigned long long)0x7ffe);   // every real step is below 0x7fff
+        __syncthreads();                                    // the histogram's room is free again
+
+        // ---- distances of the candidates, k best ---------------------------------------
+        // Every wavefront walks a quarter of the points; a candidate whose packed
+        // (distance, id) does not beat the current k-th best is dropped at once, the others
+        // wait in the wavefront's share of the buffer until the next merge.
+        const bool vec4 = rows_vec4(a.data, a.dim);
+        const int chunk = (n + kDWaves - 1) / kDWaves;
+        int at = wave * chunk;                              // next point of this wavefront (wave-uniform)
+        const int at_end = min(n, at + chunk);
+        unsigned long long pending_mask = 0;                // candidates of the 64 points loaded last
+        int mask_base = at;
+        uint32_t ncand = 0;
+        int topn = 0;
+        for (;;) {
+            unsigned long long kth = ~0ull;
+            if (topn >= a.kcap) kth = sortbuf[a.kcap - 1];
+            int mine = 0;                                   // entries this wavefront has pending
+            unsigned long long* my_slots = sortbuf + a.kcap + wave * y.quota;
+            while (mine < y.quota) {
+                if (pending_mask == 0) {
+                    if (at >= at_end) break;
+                    const int pt = at + lane;
+                    const uint32_t v = pt < at_end ? (uint32_t)s_time[pt] : 0xffffu;
+                    pending_mask = __ballot((v >> 1) <= t_lim);
+                    mask_base = at;
+                    at += kWave;
+                    ncand += (uint32_t)__popcll(pending_mask);
+                    continue;
+                }
+                // two candidates at a time: their row reads overlap
+                const int l0 = __ffsll((long long)pending_mask) - 1;
+                pending_mask &= pending_mask - 1;
+                int l1 = -1;
+                if (pending_mask && mine + 1 < y.quota) {
+                    l1 = __ffsll((long long)pending_mask) - 1;
+                    pending_mask &= pending_mask - 1;
+                }
+                const int pt0 = mask_base + l0, pt1 = l1 >= 0 ? mask_base + l1 : pt0;
+                unsigned long long e0, e1;
+                if (a.blind) {      // scored by the promoting step (:498-505), no row is read
+                    e0 = ((unsigned long long)(s_time[pt0] >> 1) << 32) | (uint32_t)(off + pt0);
+                    e1 = ((unsigned long long)(s_time[pt1] >> 1) << 32) | (uint32_t)(off + pt1);
+                } else {
+                    const float* const rows2[2] = {a.data + (off + pt0) * a.dim, a.data + (off + pt1) * a.dim};
+                    float d2[2];
+                    wave_row_dists<2>(rows2, s_q, a.dim, vec4, d2);
+                    e0 = ((unsigned long long)__builtin_bit_cast(uint32_t, d2[0]) << 32) | (uint32_t)(off + pt0);
+                    e1 = ((unsigned long long)__builtin_bit_cast(uint32_t, d2[1]) << 32) | (uint32_t)(off + pt1);
+                }
+                if (e0 < kth) { if (lane == 0) my_slots[mine] = e0; mine++; }
+                if (l1 >= 0 && e1 < kth) { if (lane == 0) my_slots[mine] = e1; mine++; }
+            }
+            for (int j = mine + lane; j < y.quota; j += kWave) my_slots[j] = ~0ull;
+            const bool more = pending_mask != 0 || at < at_end;
+            if (lane == 0) {
+                scan_tmp[8 + wave] = (uint32_t)mine;
+                scan_tmp[16 + wave] = more ? 1u : 0u;
+            }
+            // (slots between the k best held so far and the first wavefront's share)
+            for (int j = topn + tid; j < a.kcap; j += kDT) sortbuf[j] = ~0ull;
+            for (int j = a.kcap + kDWaves * y.quota + tid; j < y.sort_cap; j += kDT) sortbuf[j] = ~0ull;
+            __syncthreads();
+            int added = 0, any_more = 0;
+            for (int w2 = 0; w2 < kDWaves; w2++) { added += (int)scan_tmp[8 + w2]; any_more |= (int)scan_tmp[16 + w2]; }
+            if (added > 0) {
+                bitonic_sort_u64(sortbuf, y.sort_cap);
+                topn = min(a.kcap, topn + added);
+            } else {
+                __syncthreads();
+            }
+            if (!any_more) break;
+        }
+        if (lane == 0) atomicAdd(&misc[dCand], ncand);
+        for (int j = tid; j < a.kcap; j += kDT) part_out[j] = j < topn ? sortbuf[j] : ~0ull;
+
+        // ---- hints for the batch kernel's routing, counters -----------------------------
+        __syncthreads();
+        const unsigned long long bound = (unsigned long long)n * a.L * T;
+        unsigned long long steps = min(bound, maxw + 1);
+        if (stop) steps = min(t_stop + 1, steps);
+        if (a.stop_hint && tid == 0 && stop) {
+            const float seen_stops = a.stop_hint[2 * a.B + b];
+            const float w = 1.0f / fminf(seen_stops + 1.0f, 50.0f);
+            a.stop_hint[2 * a.B + b] = fminf(seen_stops + 1.0f, 1.0e6f);
+            a.stop_hint[b] += w * ((float)(t_stop + 1) - a.stop_hint[b]);
+            a.stop_hint[a.B + b] += w * ((float)misc[dCand] - a.stop_hint[a.B + b]);
+        }
+        if (a.counters) {
+            for (int o = 32; o > 0; o >>= 1) probes += (uint32_t)__shfl_xor((int)probes, o, kWave);
+            if (lane == 0) atomicAdd(&misc[dProbes], probes);
+            __syncthreads();
+            if (tid == 0) {
+                atomicAdd(&a.counters[(int64_t)qi * 4 + 0], (unsigned long long)n * I);
+                atomicAdd(&a.counters[(int64_t)qi * 4 + 1], (unsigned long long)misc[dCand]);
+                atomicAdd(&a.counters[(int64_t)qi * 4 + 2], (unsigned long long)misc[dProbes]);
+                atomicAdd(&a.counters[(int64_t)qi * 4 + 3], steps);
+            }
+        }
+    }
+}
+
+}  // namespace
+
+bool dense_traversal_supported(const QueryArgs& a, size_t* lds_bytes) {
+    if (!a.inv || a.ppb > 32766 || a.T < 1) return false;
+    if (a.M > 64 || a.L > 64 || a.kcap > 512 || (int64_t)a.L * a.N >= 0x7fffffffLL) return false;
+    if (dense_ipt_for(dense_max_windows(a)) == 0) return false;
+    if (dense_max_windows(a) >= 0x7fff) return false;
+    if (a.xcds < 1 || a.xcds > 32 || (int64_t)a.nq * (a.B + a.xcds) >= 0x7fffffffLL) return false;
+    const DenseLayout y = make_dense_layout(a);
+    if (lds_bytes) *lds_bytes = y.lds_bytes;
+    return y.lds_bytes <= 160 * 1024 - 512;
+}
+
+int query_dense_items(const QueryArgs& a_in, hipStream_t s) {
+    QueryArgs a = a_in;
+    const DenseLayout y = make_dense_layout(a);
+    if (y.ipt == 0) return fail(-4, "query: this shape does not fit the dense traversal kernel");
+    a.q_first = 0;
+    a.q_count = a.nq;
+    // enough resident workgroups to fill the device, each striding over its die's items
+    const int per_cu = (int)max((size_t)1, min((size_t)4, (size_t)(160 * 1024) / y.lds_bytes));
+    int64_t per_xcd = (int64_t)32 * per_cu * 2;
+    const int64_t most = a.dense_items && a.mode != 3 ? (int64_t)a.dense_cap
+                                                      : block_items(a.xcds, a.B, a.nq) / a.xcds;
+    per_xcd = max((int64_t)1, min(per_xcd, most));
+    const unsigned grid = (unsigned)(per_xcd * a.xcds);
+#define DCIH_DENSE(IPT)                                                                          \
+    do {                                                                                         \
+        static DeviceOnce once;                                                                  \
+        const int rc_attr = once.run([]() -> int {                                               \
+            DCIH_HIP(hipFuncSetAttribute((const void*)traverse_dense_kernel<IPT>,                \
+                                         hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024)); \
+            return 0;                                                                            \
+        });                                                                                      \
+        if (rc_attr) return rc_attr;                                                             \
+        hipLaunchKernelGGL((traverse_dense_kernel<IPT>), dim3(grid), dim3(kDT), y.lds_bytes, s, a, y); \
+    } while (0)
+    if (y.ipt == 9) DCIH_DENSE(9);
+    else if (y.ipt == 17) DCIH_DENSE(17);
+    else if (y.ipt == 25) DCIH_DENSE(25);
+    else DCIH_DENSE(33);
+#undef DCIH_DENSE
+    DCIH_HIP(hipGetLastError());
+    return 0;
+}
+
+}  // namespace dcih

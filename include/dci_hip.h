@@ -52,14 +52,20 @@ enum {
 /*
  * Options of dcih_set_option.  DCIH_OPT_TRAVERSAL picks the query kernel:
  * 0 = automatic (the batch kernel when the shape fits its tables, else the
- * step-by-step kernel), 1 = step-by-step kernel (one wavefront per partition,
+ * step-by-step kernel; items whose traversal needs many promotions are finished
+ * by the dense kernel), 1 = step-by-step kernel (one wavefront per partition,
  * one window per step), 2 = batch kernel (one workgroup per partition, whole
- * index ranges per epoch; errors out if the shape does not fit).  Both give the
- * same neighbours; with the batch kernel DCIH_CTR_VISITED counts the entries it
- * streamed (a superset of the reference's visits, it overshoots the stop step
- * inside its last epoch) and DCIH_CTR_PROBES its own key reads.
+ * index ranges per epoch; errors out if the shape does not fit), 3 = dense kernel
+ * (one workgroup per partition computes the promoting step of every point;
+ * errors out if the shape does not fit).  All give the same neighbours; with the
+ * batch and dense kernels DCIH_CTR_VISITED counts the entries they processed (a
+ * superset of the reference's visits: the batch kernel overshoots the stop step
+ * inside its last epoch, the dense kernel looks at every entry) and
+ * DCIH_CTR_PROBES their own key reads.  DCIH_OPT_DENSE_MIN_PROMOTIONS: under
+ * automatic choice, the number of promotions per (query, partition) from which
+ * an item goes to the dense kernel (default 384; 0 = never).
  */
-enum { DCIH_OPT_TRAVERSAL = 0 };
+enum { DCIH_OPT_TRAVERSAL = 0, DCIH_OPT_DENSE_MIN_PROMOTIONS = 1 };
 
 /* Message for the last failing call on this thread ("" if none). */
 const char* dcih_last_error(void);

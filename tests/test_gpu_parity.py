@@ -112,6 +112,24 @@ def test_segsort_matches_oracle(gpu, oracle, n, I, B):
     np.testing.assert_array_equal(si, ri)
 
 
+# one slice length inside the range of every instantiation of the LDS radix kernel
+@pytest.mark.parametrize("n", [560, 600, 1500, 2000, 2500, 3400, 4200, 5300, 5556, 6000, 8000, 9900, 11000,
+                               13000, 14500, 16000, 17858, 19000, 23000, 26000, 29000, 32000])
+def test_segsort_every_radix_configuration(gpu, oracle, n):
+    rng = np.random.default_rng(n)
+    I, B = 6, 3
+    keys = (rng.standard_normal((I, n * B - 5)) * 300 + 100).astype(np.float32)
+    keys[0, ::5] = np.round(keys[0, ::5])
+    keys[1] = np.abs(keys[1])                       # constant sign: a skipped digit
+    keys[2, ::3] = -0.0
+    keys[2, 1::3] = 0.0
+    for rep in range(2):                            # twice: the result must not depend on timing
+        sk, si = engine_segsort(keys, B)
+        rk, ri = oracle.segsort(keys, B)
+        np.testing.assert_array_equal(sk, rk)
+        np.testing.assert_array_equal(si, ri)
+
+
 def test_index_arrays_are_consistent(gpu):
     """sids, the 16-bit partition-relative ids and the inverse permutation describe
     one and the same order (checked through a query that uses all three)."""
@@ -161,15 +179,27 @@ CASES = [
     (40000, 16, 24, 2, 12, 2, 16, 10, 200, "normal"),       # step limit ends it: hundreds of promotions, large tables
     (30000, 16, 16, 2, 15, 2, 4, 50, 300, "normal"),        # L = 15: 4-bit counters with the promoted bitmap
     (30000, 16, 16, 2, 14, 3, 8, 40, 100, "normal"),        # L = 14: promoted points marked in the counters
+    (40000, 16, 24, 2, 12, 8, 16, 10, 200, "normal"),       # the step limit ends it after most of the index (dense regime)
+    (30000, 16, 16, 2, 15, 16, 4, 50, 300, "normal"),       # L = 15, several hundred promotions per partition
+    (20000, 16, 16, 3, 8, 4, 16, 100, 40, "normal"),        # three composites, k = 100
+    (6000, 16, 12, 2, 6, 3, 2, 5, 10_000, "normal"),        # narrow windows, stop by c0 >= 10k
 ]
 
 
-@pytest.mark.parametrize("traversal", ["step", "batch"])
+def _dense_fits(n, M, L, B, T, k):
+    ppb = -(-n // B)
+    return (M <= 64 and L <= 64 and ppb <= 32766 and min(k, ppb) <= 512 and
+            L * (ppb // T + 3) <= 33 * 256)
+
+
+@pytest.mark.parametrize("traversal", ["step", "batch", "dense", "auto"])
 @pytest.mark.parametrize("case", CASES, ids=[str(c[:9]) for c in CASES])
 def test_traversal_parity(gpu, oracle, case, traversal):
     n, nq, dim, M, L, B, T, k, outer, kind = case
     if traversal == "batch" and (2 * M * L > 256 or M > 64 or min(k, -(-n // B)) > 512):
         pytest.skip("shape outside the batch kernel's tables (it refuses; auto mode falls back)")
+    if traversal == "dense" and not _dense_fits(n, M, L, B, T, k):
+        pytest.skip("shape outside the dense kernel's tables (it refuses; auto mode does not route there)")
     X, Q = _data(n * 7 + T, n, nq, dim, kind)
     ids, dists, ctr, ref = _run_l1(gpu, oracle, X, Q, M, L, B, T, k, outer, traversal=traversal)
     _assert_l1(ids, dists, ctr, ref, exact_ids=(kind != "grid"), visits=(traversal == "step"))

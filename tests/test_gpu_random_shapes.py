@@ -1,4 +1,4 @@
-"""Randomised traversal parity: both query kernels against the CPU oracle on many
+"""Randomised traversal parity: all query kernels against the CPU oracle on many
 small seeded shapes, including the awkward corners (L = 1, where every visit is a
 promotion; duplicated points, where priorities tie everywhere; windows wider
 than a partition; budgets of 0 and 1 iterations; tiny max_num_candidates),
@@ -62,7 +62,7 @@ def test_random_shape(gpu, oracle, seed):
     ref = bref = None
     # "auto" may compute a traversal that provably runs dry directly; "batch" forces the
     # batch kernel and is skipped where the shape does not fit its tables
-    for traversal in ("step", "auto", "batch"):
+    for traversal in ("step", "auto", "batch", "dense"):
         dci = gpu.DCI(dim, M, L, B, T, seed=seed, traversal=traversal)
         dci.add(xd)
         ids = torch.empty((nq, k), dtype=torch.int32, device="cuda")
@@ -73,7 +73,7 @@ def test_random_shape(gpu, oracle, seed):
                                             B, T, ids.data_ptr(), dists.data_ptr(), ctr.data_ptr(),
                                             torch.cuda.current_stream().cuda_stream))
         except _capi.DCIError as e:
-            if traversal == "batch" and "does not fit" in str(e):
+            if traversal in ("batch", "dense") and "does not fit" in str(e):
                 dci.free()
                 continue
             raise
