@@ -23,6 +23,8 @@
 // points promoted up to it get their exact distances (rows read by whole
 // wavefronts) and go through a k-best filter.  Shapes that do not fit the tables
 // are left to the other kernels through the same hand-over list.
+#include <type_traits>
+
 #include "common.h"
 #include "kernels.h"
 #include "radix_core.h"
@@ -49,7 +51,7 @@ struct DenseLayout {
     int off_time;     // uint16 per point: step << 1 | lane-0 flag
     int off_sort;     // k best + pending candidates, 64-bit words
     int off_stage;    // radix staging; later the rank table, then the step histogram
-    int off_misc;
+    int off_misc, off_wlist;
     int sort_cap, quota;
     size_t lds_bytes;
 };
@@ -81,6 +83,7 @@ DenseLayout make_dense_layout(const QueryArgs& a) {
     while (y.sort_cap < a.kcap + 4 * 8) y.sort_cap <<= 1;
     y.quota = (y.sort_cap - a.kcap) / kDWaves;
     y.off_sort = o;     o += y.sort_cap * 8;
+    y.off_wlist = o;    o += kDWaves * kWave * 2;
     y.off_stage = o;    o += (y.ipt + 8) * kDT * 4;      // staging words, then the digit counters
     y.lds_bytes = (size_t)o;
     return y;
@@ -102,6 +105,7 @@ __global__ __launch_bounds__(kDT, 2) void traverse_dense_kernel(QueryArgs a, Den
     unsigned long long* sortbuf = reinterpret_cast<unsigned long long*>(smem + y.off_sort);
     uint32_t* stage = reinterpret_cast<uint32_t*>(smem + y.off_stage);
     uint16_t* rank16 = reinterpret_cast<uint16_t*>(stage);
+    uint16_t* s_wlist = reinterpret_cast<uint16_t*>(smem + y.off_wlist);   // per wavefront: 64 candidates
 
     const int tid = threadIdx.x;
     const int lane = tid & (kWave - 1);
@@ -116,6 +120,16 @@ __global__ __launch_bounds__(kDT, 2) void traverse_dense_kernel(QueryArgs a, Den
     const bool listed = a.dense_items != nullptr && a.mode != 3;
     const int64_t my_count = listed ? (int64_t)a.dense_count[xcd]
                                     : block_items(X, a.B, a.q_count) / X;
+
+    // optional phase profile: thread 0 adds the 100 MHz ticks each phase took
+    unsigned long long tick = 0ull;
+    auto phase = [&](int which) {
+        if (a.phase_ticks && tid == 0) {
+            const unsigned long long now = wall_clock64();
+            atomicAdd(&a.phase_ticks[which], now - tick);
+            tick = now;
+        }
+    };
 
     for (int64_t slot = g0; slot < my_count; slot += G) {
         int b, qi;
@@ -138,6 +152,7 @@ __global__ __launch_bounds__(kDT, 2) void traverse_dense_kernel(QueryArgs a, Den
         }
 
         // ---- set-up: query row, positioning searches (:279-297) -------------------
+        if (a.phase_ticks) tick = wall_clock64();
         if (tid < dMiscWords) misc[tid] = 0;
         for (int j = tid; j < a.dim; j += kDT) s_q[j] = a.query[(int64_t)qi * a.dim + j];
         for (int pt = tid; pt < n; pt += kDT) s_time[pt] = (uint16_t)((kNever << 1) & 0xffffu);
@@ -157,6 +172,7 @@ __global__ __launch_bounds__(kDT, 2) void traverse_dense_kernel(QueryArgs a, Den
             }
         }
         __syncthreads();
+        phase(0);
 
         unsigned long long maxw = 0;             // most windows any composite has
         for (int m = 0; m < a.M; m++) {
@@ -233,11 +249,13 @@ __global__ __launch_bounds__(kDT, 2) void traverse_dense_kernel(QueryArgs a, Den
                 if (lane == 0) { atomicOr(&misc[dOr], vor); atomicAnd(&misc[dAnd], vand); }
             }
             __syncthreads();
+            phase(1);
             // (the pads need no pass of their own: they start behind every window, every
             //  digit of theirs is the largest, and the passes are stable)
             const uint32_t varying = misc[dOr] ^ misc[dAnd];
             lds_radix_passes<kDT, IPT>(k, rp, stage, stage + IPT * kDT, scan_tmp, varying);
             __syncthreads();
+            phase(2);
             // the step of every window: its place in the sorted order
 #pragma unroll
             for (int r = 0; r < IPT; r++) {
@@ -291,6 +309,7 @@ __global__ __launch_bounds__(kDT, 2) void traverse_dense_kernel(QueryArgs a, Den
                 }
             }
             __syncthreads();
+            phase(3);
         }
         if (misc[dFail]) {      // does not fit the tables: the step-by-step kernel takes the item
             if (tid == 0) {
@@ -348,80 +367,142 @@ __global__ __launch_bounds__(kDT, 2) void traverse_dense_kernel(QueryArgs a, Den
         }
         const uint32_t t_lim = (uint32_t)min(t_stop, (unsigned long long)0x7ffe);   // every real step is below 0x7fff
         __syncthreads();                                    // the histogram's room is free again
+        phase(4);
 
         // ---- distances of the candidates, k best ---------------------------------------
         // Every wavefront walks a quarter of the points; a candidate whose packed
         // (distance, id) does not beat the current k-th best is dropped at once, the others
         // wait in the wavefront's share of the buffer until the next merge.
+        // Rows of up to 64 (128) elements are read by 16 (32) lanes each, four (two) rows
+        // per load instruction and up to four such loads in flight; the lanes' partial sums
+        // and the order in which they are added are those of wave_row_dists (the lanes a
+        // short row leaves idle there add zeros), so the distances have the same bits.
         const bool vec4 = rows_vec4(a.data, a.dim);
         const int chunk = (n + kDWaves - 1) / kDWaves;
         int at = wave * chunk;                              // next point of this wavefront (wave-uniform)
         const int at_end = min(n, at + chunk);
-        unsigned long long pending_mask = 0;                // candidates of the 64 points loaded last
-        int mask_base = at;
+        uint16_t* wl = s_wlist + wave * kWave;              // this wavefront's candidates among the 64 points loaded last
+        int list_len = 0, list_pos = 0;
         uint32_t ncand = 0;
         int topn = 0;
-        for (;;) {
-            unsigned long long kth = ~0ull;
-            if (topn >= a.kcap) kth = sortbuf[a.kcap - 1];
-            int mine = 0;                                   // entries this wavefront has pending
-            unsigned long long* my_slots = sortbuf + a.kcap + wave * y.quota;
-            while (mine < y.quota) {
-                if (pending_mask == 0) {
-                    if (at >= at_end) break;
-                    const int pt = at + lane;
-                    const uint32_t v = pt < at_end ? (uint32_t)s_time[pt] : 0xffffu;
-                    pending_mask = __ballot((v >> 1) <= t_lim);
-                    mask_base = at;
-                    at += kWave;
-                    ncand += (uint32_t)__popcll(pending_mask);
-                    continue;
+        auto run_rounds = [&](auto gtag, auto rtag) {
+            constexpr int GL = decltype(gtag)::value;       // lanes per row
+            constexpr int R = decltype(rtag)::value;        // rows per lane group in flight
+            constexpr int NG = kWave / GL;                  // lane groups
+            constexpr int RB = NG * R;                      // rows per batch
+            const int grp = lane / GL, sl = lane & (GL - 1);
+            for (;;) {
+                unsigned long long kth = ~0ull;
+                if (topn >= a.kcap) kth = sortbuf[a.kcap - 1];
+                int mine = 0;                               // entries this wavefront has pending
+                unsigned long long* my_slots = sortbuf + a.kcap + wave * y.quota;
+                for (;;) {
+                    if (list_pos >= list_len) {
+                        if (at >= at_end) break;
+                        const int pt = at + lane;
+                        const uint32_t v = pt < at_end ? (uint32_t)s_time[pt] : 0xffffu;
+                        const bool is_cand = (v >> 1) <= t_lim;
+                        const unsigned long long m = __ballot(is_cand);
+                        if (is_cand) wl[__popcll(m & ((1ull << lane) - 1ull))] = (uint16_t)pt;
+                        list_len = __popcll(m);
+                        list_pos = 0;
+                        at += kWave;
+                        ncand += (uint32_t)list_len;
+                        continue;
+                    }
+                    if (mine + RB > y.quota) break;         // no room for a whole batch: merge first
+                    int pts[R];
+                    bool valid[R];
+                    unsigned long long e[R];
+#pragma unroll
+                    for (int r = 0; r < R; r++) {
+                        const int c = list_pos + r * NG + grp;
+                        valid[r] = c < list_len;
+                        pts[r] = (int)wl[min(c, list_len - 1)];
+                    }
+                    if (a.blind) {      // scored by the promoting step (:498-505), no row is read
+#pragma unroll
+                        for (int r = 0; r < R; r++)
+                            e[r] = ((unsigned long long)(s_time[pts[r]] >> 1) << 32) | (uint32_t)(off + pts[r]);
+                    } else if (GL == kWave) {
+                        const float* rows[R];
+#pragma unroll
+                        for (int r = 0; r < R; r++) rows[r] = a.data + (off + pts[r]) * a.dim;
+                        float d[R];
+                        const float* const (&crows)[R] = rows;
+                        wave_row_dists<R>(crows, s_q, a.dim, vec4, d);
+#pragma unroll
+                        for (int r = 0; r < R; r++)
+                            e[r] = ((unsigned long long)__builtin_bit_cast(uint32_t, d[r]) << 32) | (uint32_t)(off + pts[r]);
+                    } else {
+                        typedef float v4f __attribute__((ext_vector_type(4)));
+                        float acc[R];
+                        const int j = sl * 4;
+                        v4f x[R];
+#pragma unroll
+                        for (int r = 0; r < R; r++) {
+                            acc[r] = 0.f;
+                            if (j < a.dim) x[r] = *reinterpret_cast<const v4f*>(a.data + (off + pts[r]) * a.dim + j);
+                        }
+                        if (j < a.dim) {
+                            const float q0 = s_q[j], q1 = s_q[j + 1], q2 = s_q[j + 2], q3 = s_q[j + 3];
+#pragma unroll
+                            for (int r = 0; r < R; r++) {
+                                float dd = x[r].x - q0; acc[r] = __builtin_fmaf(dd, dd, acc[r]);
+                                dd = x[r].y - q1; acc[r] = __builtin_fmaf(dd, dd, acc[r]);
+                                dd = x[r].z - q2; acc[r] = __builtin_fmaf(dd, dd, acc[r]);
+                                dd = x[r].w - q3; acc[r] = __builtin_fmaf(dd, dd, acc[r]);
+                            }
+                        }
+#pragma unroll
+                        for (int r = 0; r < R; r++) {
+                            float v = acc[r];
+#pragma unroll
+                            for (int o = GL / 2; o > 0; o >>= 1) v += __shfl_xor(v, o, kWave);
+                            e[r] = ((unsigned long long)__builtin_bit_cast(uint32_t, sqrtf(v)) << 32) | (uint32_t)(off + pts[r]);
+                        }
+                    }
+#pragma unroll
+                    for (int r = 0; r < R; r++) {
+                        const bool keep = valid[r] && sl == 0 && e[r] < kth;
+                        const unsigned long long m = __ballot(keep);
+                        if (keep) my_slots[mine + __popcll(m & ((1ull << lane) - 1ull))] = e[r];
+                        mine += __popcll(m);
+                    }
+                    list_pos += RB;
                 }
-                // two candidates at a time: their row reads overlap
-                const int l0 = __ffsll((long long)pending_mask) - 1;
-                pending_mask &= pending_mask - 1;
-                int l1 = -1;
-                if (pending_mask && mine + 1 < y.quota) {
-                    l1 = __ffsll((long long)pending_mask) - 1;
-                    pending_mask &= pending_mask - 1;
+                for (int j = mine + lane; j < y.quota; j += kWave) my_slots[j] = ~0ull;
+                const bool more = list_pos < list_len || at < at_end;
+                if (lane == 0) {
+                    scan_tmp[8 + wave] = (uint32_t)mine;
+                    scan_tmp[16 + wave] = more ? 1u : 0u;
                 }
-                const int pt0 = mask_base + l0, pt1 = l1 >= 0 ? mask_base + l1 : pt0;
-                unsigned long long e0, e1;
-                if (a.blind) {      // scored by the promoting step (:498-505), no row is read
-                    e0 = ((unsigned long long)(s_time[pt0] >> 1) << 32) | (uint32_t)(off + pt0);
-                    e1 = ((unsigned long long)(s_time[pt1] >> 1) << 32) | (uint32_t)(off + pt1);
-                } else {
-                    const float* const rows2[2] = {a.data + (off + pt0) * a.dim, a.data + (off + pt1) * a.dim};
-                    float d2[2];
-                    wave_row_dists<2>(rows2, s_q, a.dim, vec4, d2);
-                    e0 = ((unsigned long long)__builtin_bit_cast(uint32_t, d2[0]) << 32) | (uint32_t)(off + pt0);
-                    e1 = ((unsigned long long)__builtin_bit_cast(uint32_t, d2[1]) << 32) | (uint32_t)(off + pt1);
-                }
-                if (e0 < kth) { if (lane == 0) my_slots[mine] = e0; mine++; }
-                if (l1 >= 0 && e1 < kth) { if (lane == 0) my_slots[mine] = e1; mine++; }
-            }
-            for (int j = mine + lane; j < y.quota; j += kWave) my_slots[j] = ~0ull;
-            const bool more = pending_mask != 0 || at < at_end;
-            if (lane == 0) {
-                scan_tmp[8 + wave] = (uint32_t)mine;
-                scan_tmp[16 + wave] = more ? 1u : 0u;
-            }
-            // (slots between the k best held so far and the first wavefront's share)
-            for (int j = topn + tid; j < a.kcap; j += kDT) sortbuf[j] = ~0ull;
-            for (int j = a.kcap + kDWaves * y.quota + tid; j < y.sort_cap; j += kDT) sortbuf[j] = ~0ull;
-            __syncthreads();
-            int added = 0, any_more = 0;
-            for (int w2 = 0; w2 < kDWaves; w2++) { added += (int)scan_tmp[8 + w2]; any_more |= (int)scan_tmp[16 + w2]; }
-            if (added > 0) {
-                bitonic_sort_u64(sortbuf, y.sort_cap);
-                topn = min(a.kcap, topn + added);
-            } else {
+                // (slots between the k best held so far and the first wavefront's share)
+                for (int j = topn + tid; j < a.kcap; j += kDT) sortbuf[j] = ~0ull;
+                for (int j = a.kcap + kDWaves * y.quota + tid; j < y.sort_cap; j += kDT) sortbuf[j] = ~0ull;
                 __syncthreads();
+                int added = 0, any_more = 0;
+                for (int w2 = 0; w2 < kDWaves; w2++) { added += (int)scan_tmp[8 + w2]; any_more |= (int)scan_tmp[16 + w2]; }
+                if (added > 0) {
+                    bitonic_sort_u64(sortbuf, y.sort_cap);
+                    topn = min(a.kcap, topn + added);
+                } else {
+                    __syncthreads();
+                }
+                if (!any_more) break;
             }
-            if (!any_more) break;
+        };
+        {
+            using std::integral_constant;
+            if (vec4 && !a.blind && a.dim <= 64 && y.quota >= 16) run_rounds(integral_constant<int, 16>{}, integral_constant<int, 4>{});
+            else if (vec4 && !a.blind && a.dim <= 64) run_rounds(integral_constant<int, 16>{}, integral_constant<int, 2>{});
+            else if (vec4 && !a.blind && a.dim <= 128) run_rounds(integral_constant<int, 32>{}, integral_constant<int, 4>{});
+            else run_rounds(integral_constant<int, 64>{}, integral_constant<int, 2>{});
         }
         if (lane == 0) atomicAdd(&misc[dCand], ncand);
         for (int j = tid; j < a.kcap; j += kDT) part_out[j] = j < topn ? sortbuf[j] : ~0ull;
+        phase(5);
+        if (a.phase_ticks && tid == 0) atomicAdd(&a.phase_ticks[9], 1ull);
 
         // ---- hints for the batch kernel's routing, counters -----------------------------
         __syncthreads();

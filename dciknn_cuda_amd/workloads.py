@@ -86,3 +86,40 @@ def c5_queries(nq=10_000, dim=64):
 def directions(config, num_indices, dim):
     """Unnormalised N(0,1) direction draws for a config (stream 4)."""
     return torch.randn(num_indices, dim, generator=_gen(config, 4))
+
+
+def exact_knn(X, Q, k, query_chunk=256, point_chunk=1 << 20):
+    """Exact k nearest neighbours (ids, ascending by distance) of the rows of Q among the
+    rows of X, on the device the tensors live on: recall ground truth.  A fast
+    ||x||^2 - 2 q.x pass over blocks of points picks a pool of candidates per block
+    (the matrix product's rounding and very long top-k rows are both kept out of the
+    answer that way), whose distances are then recomputed in float64 for the final cut."""
+    n = X.shape[0]
+    pool = min(n, max(2 * k, k + 64))
+    xn = (X * X).sum(1)
+    out = []
+    for q0 in range(0, Q.shape[0], query_chunk):
+        q = Q[q0:q0 + query_chunk]
+        cands = []
+        for p0 in range(0, n, point_chunk):
+            xb = X[p0:p0 + point_chunk]
+            d2 = xn[None, p0:p0 + point_chunk] - 2.0 * (q @ xb.T)
+            cands.append(d2.topk(min(pool, xb.shape[0]), dim=1, largest=False).indices + p0)
+        cand = torch.cat(cands, 1)
+        best = None
+        for c0 in range(0, cand.shape[1], 4096):       # bounded memory for the float64 pass
+            cc = cand[:, c0:c0 + 4096]
+            d = (X[cc].double() - q[:, None, :].double()).norm(dim=2)
+            if best is not None:
+                d = torch.cat([best[0], d], 1)
+                cc = torch.cat([best[1], cc], 1)
+            top = d.topk(min(k, d.shape[1]), dim=1, largest=False)
+            best = (top.values, torch.gather(cc, 1, top.indices))
+        out.append(best[1])
+    return torch.cat(out)
+
+
+def recall_at_k(ids, truth):
+    """Fraction of the true neighbours (rows of `truth`) found in the same rows of `ids`."""
+    hit = (ids.long()[:, :, None] == truth.long()[:, None, :]).any(2).float().sum().item()
+    return hit / truth.numel()
