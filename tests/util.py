@@ -46,3 +46,15 @@ def engine_segsort(keys, block_size):
                                          torch.cuda.current_stream().cuda_stream))
     torch.cuda.synchronize()
     return sk.cpu().numpy(), si.cpu().numpy()
+
+
+def dense_fits(n, M, L, B, T, k):
+    """Shapes the dense traversal kernel's tables take (it refuses the others)."""
+    ppb = -(-n // B)
+    return (M <= 64 and L <= 64 and ppb <= 32766 and min(k, ppb) <= 512 and
+            L * (ppb // T + 3) <= 33 * 256)
+
+
+def batch_fits(n, M, L, B, k):
+    """Shapes the batch traversal kernel's tables take (it refuses the others)."""
+    return 2 * M * L <= 256 and M <= 64 and min(k, -(-n // B)) <= 512 and -(-n // B) <= 65536
