@@ -1,19 +1,34 @@
 """Benchmark of the Prioritized DCI hot path on one MI355X.
 
     python bench.py [--gpus 1] [--steps K] [--warmup W] [--config c2]
-                    [--bs B --ts T --outer O] [--nq NQ] [--no-cpu]
+                    [--bs B --ts T --outer O] [--nq NQ] [--no-cpu] [--no-extras]
 
 A step is one pass of the query path (query projection, traversal, exact
 distances, top-k) over the whole seeded query batch of the workload, with the
 index built and all inputs resident in HBM.  The build (projection + segmented
-sort) is timed separately and reported as build_points_per_s.  Prints ONE JSON
-line: value = queries/s; recall_at_k against exact brute force; per_query = exact
-traversal counters of the reference algorithm on a query sample; kernel_ms and
-build = HIP-event times inside the library; roofline = the traversal kernel's
-algorithmic bytes (by the reference's 8-byte index entries) over its time, with
-the measured HBM traffic beside it; cpu_baseline = the CPU restatement of the
-reference algorithm on this box's host cores, on a bounded query sample; blind =
-the same batch queried blind (candidate ids by promoting step, no distances).
+sort) is timed separately and reported as build_points_per_s; for the
+incremental workload (c5) the index is grown by appends, each timed, and the
+steps run on the final index.  Prints ONE JSON line:
+
+  value          queries/s over the timed steps
+  recall_at_k    against exact k-NN, recall_ok = the workload's target is met
+  per_query      exact traversal counters of the reference algorithm (step-by-step
+                 kernel = oracle counts) on a query sample, and what the timed
+                 kernels themselves streamed
+  kernel_ms      HIP-event times of the query kernels inside the library
+  build          HIP-event times of projection and sort, their HBM fractions
+  roofline       the kernel that took most of the step, against the limit that binds
+                 it: `frac` is always achieved / peak of that limit (<= 1).  For the
+                 batch traversal kernel the limit is vector-ALU issue (lane
+                 instructions), for the dense traversal kernel HBM bytes (candidate
+                 rows + index slices); the figure by the reference's 8-byte index
+                 entries is kept as contract_bytes_* and is not a bound.  `traffic`
+                 = HBM bytes per launch from profiles/hbm_traffic.json (rocprofv3
+                 counter runs of this file), null when that file has no entry for
+                 the configuration and setting being run
+  cpu_baseline   the CPU restatement of the reference algorithm on this box's host
+                 cores on a bounded sample of the same workload
+  first_call, outer_sweep, blind   extra measurements outside the timed steps
 """
 import argparse
 import json
@@ -25,24 +40,34 @@ ROOT = os.path.dirname(os.path.abspath(__file__))
 sys.path.insert(0, ROOT)
 
 HBM_PEAK_GBS = 8000.0   # MI355X HBM3E
+# vector-ALU issue peak: 256 CUs x 4 SIMDs x 16 lanes x 2.4 GHz lane instructions per second
+VALU_PEAK_GOPS = 256 * 4 * 16 * 2.4
+# lane instructions the batch kernel cannot do without per streamed index entry: its share
+# of the 16-byte id read, the id's extraction, the counter's address, the LDS update
+MIN_INSTR_PER_ENTRY = 4.0
 
-# HBM bytes per launch of the batch traversal kernel on the default workload and
-# setting (C2 at TUNED["c2"], all 10000 queries), from rocprofv3 --pmc FETCH_SIZE and
-# WRITE_SIZE, each scaled by what the same counter reads for a 1 GiB device copy
-# (2.000 and 1.000); the counter runs are summarised in profiles/bench_c2_hbm_traffic.txt.
-# Counters cannot be read from inside this process, so the figure is a constant
-# tied to that exact configuration and omitted for any other.
-MEASURED_TRAFFIC_C2_DEFAULT = 49.3e9
-
-# (block_size, thread_size, num_outer_iterations) used when none are given:
-# the fastest setting found with recall@k >= 0.95 on that workload.
+# (block_size, thread_size, num_outer_iterations) used when none are given: the fastest
+# setting found that meets the workload's recall target (RECALL_TARGET; c5 has none and
+# runs at a setting whose partitions stay within 16-bit positions up to 20M points).
 TUNED = {
     "c1": dict(bs=100, ts=10, outer=5000),
     "c2": dict(bs=56, ts=2, outer=500),
-    "c3": dict(bs=1000, ts=16, outer=500),
-    "c4": dict(bs=100, ts=10, outer=500),
-    "c5": dict(bs=640, ts=2, outer=500),
+    "c3": dict(bs=500, ts=32, outer=530),
+    "c4": dict(bs=100, ts=16, outer=500),
+    "c5": dict(bs=640, ts=8, outer=500),
 }
+RECALL_TARGET = {"c1": 0.95, "c2": 0.95, "c3": 0.9, "c4": 0.95, "c5": None}
+# queries per leg that would otherwise take minutes on the large workloads
+LEG_QUERIES = {
+    "c1": dict(recall=500, counters=500, cpu=500, blind=500),
+    "c2": dict(recall=10_000, counters=512, cpu=2048, blind=10_000),
+    "c3": dict(recall=1024, counters=32, cpu=768, blind=64),
+    "c4": dict(recall=5000, counters=256, cpu=512, blind=1000),
+    "c5": dict(recall=1024, counters=32, cpu=512, blind=256, growth=1024),
+}
+# the CPU baseline of the two 10M+ workloads runs on the first CPU_SAMPLE_POINTS points
+# with block_size scaled to keep the points per partition; its rate is scaled to full size
+CPU_SAMPLE_POINTS = 1_000_000
 
 
 def parse():
@@ -55,14 +80,12 @@ def parse():
     p.add_argument("--ts", type=int)
     p.add_argument("--outer", type=int)
     p.add_argument("--nq", type=int, help="use only the first NQ queries")
-    p.add_argument("--n", type=int, help="override the number of data points")
-    p.add_argument("--cpu-queries", type=int, default=2048,
-                   help="queries in the CPU baseline sample")
+    p.add_argument("--n", type=int, help="override the number of data points (c5: per batch)")
     p.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
+    p.add_argument("--no-extras", action="store_true",
+                   help="skip first_call, outer_sweep and blind (profiling runs)")
     p.add_argument("--build-reps", type=int, default=3)
-    p.add_argument("--counter-queries", type=int, default=512,
-                   help="queries whose exact traversal counters are taken (step-by-step kernel)")
-    p.add_argument("--traversal", default="auto", choices=["auto", "step", "batch"])
+    p.add_argument("--traversal", default="auto", choices=["auto", "step", "batch", "dense"])
     p.add_argument("--c5-batches", type=int, default=20, help="batches of the incremental workload")
     p.add_argument("--copy-calibration", action="store_true",
                    help="also run a plain 1 GiB device copy (known HBM traffic) so that "
@@ -70,76 +93,20 @@ def parse():
     return p.parse_args()
 
 
-def exact_knn_gpu(X, Q, k, chunk=1024):
-    """Exact k-NN by chunked fp32 matmul on the GPU (recall ground truth)."""
-    import torch
-    xn = (X * X).sum(1)
-    out = []
-    for s in range(0, Q.shape[0], chunk):
-        q = Q[s:s + chunk]
-        d2 = xn[None, :] - 2.0 * (q @ X.T)
-        out.append(d2.topk(k, dim=1, largest=False).indices)
-    return torch.cat(out)
-
-
-def recall_at_k(ids, gt):
-    hit = (ids[:, :, None] == gt[:, None, :]).any(2).float().sum().item()
-    return hit / gt.numel()
-
-
-def run_c5(a):
-    """Incremental workload: batches of 1M x 64 N(0,1) rows appended one after the
-    other, the fixed query batch run after each; one JSON line with per-size figures."""
-    import numpy as np
-    import torch
-    from dciknn_cuda_amd import build as engine_build
-    engine_build.ensure_built()      # loads what is built; compiles only in a tree without libraries
-    import dciknn_cuda_amd as D
-    from dciknn_cuda_amd import workloads
-    cfg = dict(TUNED["c5"])
-    for key in ("bs", "ts", "outer"):
-        if getattr(a, key) is not None:
-            cfg[key] = getattr(a, key)
-    shape = workloads.SHAPES[5]
-    n_batch = a.n or shape["n"]
-    nq = a.nq or shape["nq"]
-    M, L, k, dim = shape["m"], shape["l"], shape["k"], 64
-    Qd = workloads.c5_queries(nq).cuda()
-    dci = D.DCI(dim, M, L, cfg["bs"], cfg["ts"], seed=4)
-    rows = []
-    all_x = []
-    for b in range(a.c5_batches):
-        xb = workloads.c5_batch(b, n=n_batch).cuda()
-        all_x.append(xb)
-        torch.cuda.synchronize()
-        t0 = time.perf_counter()
-        dci.append(xb)
-        torch.cuda.synchronize()
-        t_add = time.perf_counter() - t0
-        dci.query(Qd, k, cfg["outer"], return_int=True)          # warm-up (hints, workspace)
-        torch.cuda.synchronize()
-        t0 = time.perf_counter()
-        ids, dists = dci.query(Qd, k, cfg["outer"], return_int=True)
-        torch.cuda.synchronize()
-        t_q = time.perf_counter() - t0
-        X = torch.cat(all_x)
-        gt = exact_knn_gpu(X, Qd[:256], k)
-        rec = recall_at_k(ids[:256].long(), gt)
-        del X
-        rows.append(dict(points=dci.num_points, append_ms=t_add * 1e3,
-                         new_points_per_s=n_batch / t_add, total_points_per_s=dci.num_points / t_add,
-                         queries_per_s=nq / t_q, recall_at_k=rec))
-    out = {"metric": "queries/sec; index build points/sec (incremental)", "value": rows[-1]["queries_per_s"],
-           "unit": "queries/s", "n_gpus": 1, "steps": 1, "warmup": 1,
-           "ms_per_step": nq / rows[-1]["queries_per_s"] * 1e3, "higher_is_better": True,
-           "scaling": "weak", "vs_baseline": None, "dtype": "f32", "data": "synthetic",
-           "config": {"workload": "C5: %d appends of %d x 64 fp32 N(0,1), %d queries, m=%d L=%d k=%d"
-                                  % (a.c5_batches, n_batch, nq, M, L, k),
-                      "block_size": cfg["bs"], "thread_size": cfg["ts"],
-                      "num_outer_iterations": cfg["outer"]},
-           "build_points_per_s": rows[-1]["total_points_per_s"], "per_size": rows,
-           "roofline": None, "cpu_baseline": None}
-    print(json.dumps(out))
+def load_traffic(config, cfg, traversal, n, nq):
+    """HBM bytes per launch of the dominant kernel from the committed counter summary."""
+    path = os.path.join(ROOT, "profiles", "hbm_traffic.json")
+    try:
+        with open(path) as f:
+            table = json.load(f)
+    except (OSError, ValueError):
+        return None
+    for row in table.get("runs", []):
+        if (row.get("config") == config and row.get("bs") == cfg["bs"] and row.get("ts") == cfg["ts"]
+                and row.get("outer") == cfg["outer"] and row.get("traversal", "auto") == traversal
+                and row.get("points") == n and row.get("queries") == nq):
+            return row
+    return None
 
 
 def main():
@@ -158,25 +125,28 @@ def main():
     import dciknn_cuda_amd as D
     from dciknn_cuda_amd import _capi, workloads
 
-    if a.config == "c5":
-        return run_c5(a)
-    cfg = dict(TUNED[a.config])
+    def say(*msg):
+        print("[bench]", *msg, file=sys.stderr, flush=True)
+
+    config = a.config
+    cfg = dict(TUNED[config])
     for key in ("bs", "ts", "outer"):
         if getattr(a, key) is not None:
             cfg[key] = getattr(a, key)
-    shape = dict(workloads.SHAPES[int(a.config[1])])
-    if a.n:
-        shape["n"] = a.n
-    gen = getattr(workloads, a.config)
-    X, Q = gen(n=shape["n"], nq=shape["nq"])
-    if a.nq:
-        Q = Q[:a.nq].contiguous()
-    N, dim = X.shape
-    nq = Q.shape[0]
-    M, L, k = shape["m"], shape["l"], shape["k"]
+    shape = dict(workloads.SHAPES[int(config[1])])
+    legs = LEG_QUERIES[config]
+    M, L, k, dim = shape["m"], shape["l"], shape["k"], shape["dim"]
     I = M * L
-    Xd, Qd = X.cuda(), Q.cuda()
-    torch.cuda.synchronize()
+    outer = cfg["outer"]
+
+    dci = D.DCI(dim, M, L, cfg["bs"], cfg["ts"], seed=4, traversal=a.traversal)
+    lib = dci._lib
+    _capi.check(lib.dcih_profile(dci._dci_inst, 1))
+    tms = (_capi.ctypes.c_float * _capi.NUM_TIMERS)()
+
+    def timers():
+        _capi.check(lib.dcih_last_timings(dci._dci_inst, tms))   # waits for the call's events
+        return [float(v) for v in tms]
 
     if a.copy_calibration:
         src = torch.empty(1 << 28, dtype=torch.float32, device="cuda").normal_()
@@ -186,161 +156,305 @@ def main():
         torch.cuda.synchronize()
         del src, dst
 
-    dci = D.DCI(dim, M, L, cfg["bs"], cfg["ts"], seed=4, traversal=a.traversal)
-    lib = dci._lib
-    _capi.check(lib.dcih_profile(dci._dci_inst, 1))
-    tms = (_capi.ctypes.c_float * _capi.NUM_TIMERS)()
+    # ---- data and build ---------------------------------------------------------
+    per_size = None
+    if config == "c5":
+        n_batch = a.n or shape["n"]
+        Q = workloads.c5_queries(shape["nq"])
+        if a.nq:
+            Q = Q[:a.nq].contiguous()
+        Qd = Q.cuda()
+        nq = Q.shape[0]
+        Xd = torch.empty((a.c5_batches * n_batch, dim), dtype=torch.float32, device="cuda")
+        X_cpu_sample = None
+        per_size = []
+        Qg = Qd[:min(nq, legs["growth"])].contiguous()     # the queries run after every append
+        for b in range(a.c5_batches):
+            xb_host = workloads.c5_batch(b, n=n_batch)
+            if b == 0:
+                X_cpu_sample = xb_host
+            xb = xb_host.cuda()
+            Xd[b * n_batch:(b + 1) * n_batch] = xb
+            torch.cuda.synchronize()
+            t0 = time.perf_counter()
+            dci.append(xb)
+            torch.cuda.synchronize()
+            t_add = time.perf_counter() - t0
+            tt = timers()
+            dci.query(Qg, k, outer, return_int=True)          # warm-up (hints, workspace)
+            torch.cuda.synchronize()
+            t0 = time.perf_counter()
+            ids, _ = dci.query(Qg, k, outer, return_int=True)
+            torch.cuda.synchronize()
+            t_q = time.perf_counter() - t0
+            nrec = min(Qg.shape[0], 256)
+            truth = workloads.exact_knn(Xd[:(b + 1) * n_batch], Qg[:nrec], k)
+            per_size.append(dict(points=dci.num_points, append_ms=t_add * 1e3,
+                                 project_ms=tt[_capi.T_PROJECT], segsort_ms=tt[_capi.T_SEGSORT],
+                                 new_points_per_s=n_batch / t_add,
+                                 total_points_per_s=dci.num_points / t_add,
+                                 queries_per_s=Qg.shape[0] / t_q, queries=Qg.shape[0],
+                                 recall_at_k=workloads.recall_at_k(ids[:nrec], truth)))
+            say("c5 batch", b, "append %.2f ms, %.0f queries/s" % (t_add * 1e3, Qg.shape[0] / t_q))
+        N = dci.num_points
+        Xd = Xd[:N]
+        appends = [r["append_ms"] for r in per_size]
+        build_wall = appends[-1] * 1e-3
+        build_cold = appends[0] * 1e-3
+        proj_t, sort_t = per_size[-1]["project_ms"], per_size[-1]["segsort_ms"]
+        new_rows = n_batch
+        workload_text = "C5: %d appends of %d x %d fp32 N(0,1), %d queries, m=%d L=%d k=%d" % (
+            a.c5_batches, n_batch, dim, nq, M, L, k)
+    else:
+        if a.n:
+            shape["n"] = a.n
+        X, Q = getattr(workloads, config)(n=shape["n"], nq=shape["nq"])
+        if a.nq:
+            Q = Q[:a.nq].contiguous()
+        N, nq = X.shape[0], Q.shape[0]
+        Xd, Qd = X.cuda(), Q.cuda()
+        X_cpu_sample = X[:CPU_SAMPLE_POINTS] if N > 2 * CPU_SAMPLE_POINTS else X
+        del X
+        torch.cuda.synchronize()
+        build_s, proj_ms, sort_ms = [], [], []
+        for rep in range(a.build_reps + 1):
+            dci.clear() if dci.num_points else None
+            torch.cuda.synchronize()
+            t0 = time.perf_counter()
+            dci.add(Xd)
+            torch.cuda.synchronize()
+            t1 = time.perf_counter()
+            tt = timers()
+            if rep == 0:   # first add of the handle: allocates its arrays, loads code objects
+                build_cold = t1 - t0
+            else:          # clear + add on the same handle: steady-state rebuild
+                build_s.append(t1 - t0)
+                proj_ms.append(tt[_capi.T_PROJECT])
+                sort_ms.append(tt[_capi.T_SEGSORT])
+        build_wall = float(np.median(build_s))
+        proj_t, sort_t = float(np.median(proj_ms)), float(np.median(sort_ms))
+        new_rows = N
+        workload_text = "%s: %d pts x %d fp32, %d queries, m=%d L=%d k=%d" % (
+            config.upper(), N, dim, nq, M, L, k)
+    say("built", N, "points; build %.3f ms" % (build_wall * 1e3))
 
-    # ---- build: projection + segmented sort --------------------------------
-    build_s, proj_ms, sort_ms = [], [], []
-    for rep in range(a.build_reps + 1):
-        dci.clear() if dci.num_points else None
+    # ---- first call of this query shape: nothing learnt about where traversals stop ----
+    first_call = None
+    if not a.no_extras:
+        dci.query(Qd, k, outer)                  # workspace and kernel attributes in place
+        _capi.check(lib.dcih_set_option(dci._dci_inst, _capi.OPT_FORGET_HINTS, 0))
         torch.cuda.synchronize()
         t0 = time.perf_counter()
-        dci.add(Xd)
+        dci.query(Qd, k, outer, return_int=True)
         torch.cuda.synchronize()
-        t1 = time.perf_counter()
-        _capi.check(lib.dcih_last_timings(dci._dci_inst, tms))
-        if rep == 0:   # first add of the handle: allocates its arrays, loads code objects
-            build_cold = t1 - t0
-        else:          # clear + add on the same handle: steady-state rebuild
-            build_s.append(t1 - t0)
-            proj_ms.append(tms[_capi.T_PROJECT])
-            sort_ms.append(tms[_capi.T_SEGSORT])
-    build_wall = float(np.median(build_s))
-    proj_t, sort_t = float(np.median(proj_ms)), float(np.median(sort_ms))
+        t_first = time.perf_counter() - t0
+        first_call = dict(queries_per_s=nq / t_first, ms=t_first * 1e3,
+                          note="same batch with the stop-step hints forgotten (they size the batch "
+                               "kernel's epochs and are learnt from earlier queries; results do not depend on them)")
+        _capi.check(lib.dcih_set_option(dci._dci_inst, _capi.OPT_FORGET_HINTS, 0))
 
-    # ---- query: warmup, then K timed steps ----------------------------------
+    # ---- query: warmup, then K timed steps ----------------------------------------
     for _ in range(a.warmup):
-        dci.query(Qd, k, cfg["outer"])
-    trav_ms, merge_ms, qproj_ms = [], [], []
+        dci.query(Qd, k, outer)
+    tsum = np.zeros(_capi.NUM_TIMERS)
     torch.cuda.synchronize()
     t0 = time.perf_counter()
     for _ in range(a.steps):
-        ids, dists = dci.query(Qd, k, cfg["outer"], return_int=True)
-        _capi.check(lib.dcih_last_timings(dci._dci_inst, tms))   # waits for this step's events
-        trav_ms.append(tms[_capi.T_TRAVERSE])
-        merge_ms.append(tms[_capi.T_MERGE])
-        qproj_ms.append(tms[_capi.T_QPROJECT])
+        ids, dists = dci.query(Qd, k, outer, return_int=True)
+        tsum += np.maximum(np.array(timers()), 0.0)
     torch.cuda.synchronize()
     t1 = time.perf_counter()
     ms_per_step = (t1 - t0) * 1e3 / a.steps
     qps = nq / (ms_per_step * 1e-3)
+    tavg = tsum / a.steps
+    trav_ms, batch_ms, dense_ms = tavg[_capi.T_TRAVERSE], tavg[_capi.T_BATCH], tavg[_capi.T_DENSE]
+    say("%.0f queries/s, traverse %.2f ms (batch %.2f, dense %.2f)" % (qps, trav_ms, batch_ms, dense_ms))
 
-    # ---- outside the timed region: recall and traversal counters -------------
-    gt = exact_knn_gpu(Xd, Qd, k)
-    recall = recall_at_k(ids.long(), gt)
-    # what the kernel that was timed actually streamed / probed
-    _, _, ctr = dci.query(Qd, k, cfg["outer"], return_int=True, return_counters=True)
+    # ---- outside the timed region: recall and traversal counters ---------------------
+    nrec = min(nq, legs["recall"])
+    truth = workloads.exact_knn(Xd, Qd[:nrec].contiguous(), k)
+    recall = workloads.recall_at_k(ids[:nrec], truth)
+    target = RECALL_TARGET[config]
+    say("recall@%d %.4f on %d queries" % (k, recall, nrec))
+    # what the kernels that were timed streamed / probed themselves
+    say("counters of the timed kernels")
+    _, _, ctr = dci.query(Qd, k, outer, return_int=True, return_counters=True)
     torch.cuda.synchronize()
     own = ctr.double().mean(0).cpu().numpy()
     # exact counters of the reference algorithm (identical to the oracle's: the parity
     # tests check that) from the step-by-step kernel on a sample of the queries
-    nqc = min(nq, a.counter_queries)
+    nqc = min(nq, legs["counters"])
+    say("exact counters from the step-by-step kernel on", nqc, "queries")
     dci.set_traversal("step")
-    _, _, ctr = dci.query(Qd[:nqc].contiguous(), k, cfg["outer"], return_int=True, return_counters=True)
+    _, _, ctr = dci.query(Qd[:nqc].contiguous(), k, outer, return_int=True, return_counters=True)
     torch.cuda.synchronize()
     dci.set_traversal(a.traversal)
-    cm = ctr.double().mean(0).cpu().numpy()
-    V, C, S, steps_q = (float(v) for v in cm)
+    V, C, S, steps_q = (float(v) for v in ctr.double().mean(0).cpu().numpy())
 
-    # ---- blind querying of the same shape (outside the headline's timed region) ----
-    # no distances: per query the first min(10k, outer) promoted candidates by promoting step
-    bids, _ = dci.query(Qd, k, cfg["outer"], blind=True, return_int=True)
-    torch.cuda.synchronize()
-    t0 = time.perf_counter()
-    for _ in range(a.steps):
-        bids, _ = dci.query(Qd, k, cfg["outer"], blind=True, return_int=True)
-    torch.cuda.synchronize()
-    blind_ms = (time.perf_counter() - t0) * 1e3 / a.steps
-    hit = (gt.unsqueeze(2) == bids.long().unsqueeze(1)).any(2).float().mean().item()
-    blind = dict(queries_per_s=nq / (blind_ms * 1e-3), ms_per_step=blind_ms,
-                 slots_per_query=int(bids.shape[1]), true_neighbours_among_slots=hit)
+    # ---- roofline of the kernel that took most of the step ----------------------------
+    # By the reference's layout a query moves: its row, 8 bytes (key, id) per search probe and
+    # per visited entry, one data row per promoted point, k results.  That figure is kept for
+    # comparison only: this engine stores ids apart from keys, 2 bytes each, and an XCD works
+    # on one partition at a time so most entries come from its L2.
+    contract_bytes = 4 * dim + 8 * S + 8 * V + 4 * dim * C + 8 * k
+    ppb = -(-N // cfg["bs"])
+    if a.traversal == "step":
+        kernel, launch_ms = "traverse_kernel", trav_ms
+    elif dense_ms > batch_ms:
+        kernel, launch_ms = "traverse_dense_kernel", dense_ms
+    elif batch_ms > 0:
+        kernel, launch_ms = "traverse_block_kernel", batch_ms
+    else:   # neither traversal kernel ran: the traversal provably runs dry and the ranking is computed directly
+        kernel, launch_ms = "exact_dists_kernel + segmented sort", trav_ms
+    # bytes the launch has to bring from HBM in this layout: the index slices once (keys,
+    # 16-bit ids, 16-bit inverse positions), per query its row, the rows of its candidates and
+    # its per-partition result lists
+    hbm_bytes = 8.0 * I * N + nq * (4.0 * dim + 4.0 * dim * C + 8.0 * min(k, ppb) * cfg["bs"])
+    hbm_gbs = hbm_bytes / (launch_ms * 1e-3) / 1e9
+    valu_ops = MIN_INSTR_PER_ENTRY * float(own[0]) * nq
+    valu_gops = valu_ops / (launch_ms * 1e-3) / 1e9
+    if kernel == "traverse_block_kernel":
+        roofline = dict(bound="valu", kernel=kernel, achieved=valu_gops, peak=VALU_PEAK_GOPS,
+                        unit="G lane-instr/s", frac=valu_gops / VALU_PEAK_GOPS,
+                        model="%.0f lane instructions per index entry streamed x %.4g entries per launch"
+                              % (MIN_INSTR_PER_ENTRY, float(own[0]) * nq))
+    else:
+        roofline = dict(bound="hbm", kernel=kernel, achieved=hbm_gbs, peak=HBM_PEAK_GBS,
+                        unit="GB/s", frac=hbm_gbs / HBM_PEAK_GBS,
+                        model="index slices once (8 B per entry) + per query its row, %.0f candidate "
+                              "rows of %d B and its per-partition result lists" % (C, 4 * dim))
+    roofline.update(avg_launch_ms=launch_ms, hbm_bytes_per_launch=hbm_bytes, hbm_gbs=hbm_gbs,
+                    hbm_frac=hbm_gbs / HBM_PEAK_GBS, valu_min_lane_instr_per_launch=valu_ops,
+                    valu_frac=valu_gops / VALU_PEAK_GOPS,
+                    contract_bytes_per_launch=contract_bytes * nq,
+                    contract_bytes_gbs=contract_bytes * nq / (launch_ms * 1e-3) / 1e9,
+                    contract_note="contract_bytes_* prices every visit at the reference's 8 bytes per "
+                                  "(key, id) entry; it is not a bound for this layout and may exceed the HBM peak")
+    prof = load_traffic(config, cfg, a.traversal, N, nq)
+    roofline["traffic"] = prof["fetch_bytes"] + prof["write_bytes"] if prof else None
+    if prof:
+        roofline["traffic_source"] = {key: prof[key] for key in prof if key not in ("fetch_bytes", "write_bytes")}
+        roofline["traffic_fetch_bytes"], roofline["traffic_write_bytes"] = prof["fetch_bytes"], prof["write_bytes"]
+        if "valu_issue_frac" in prof:
+            roofline["valu_issue_frac_profiled"] = prof["valu_issue_frac"]
 
-    # Algorithmic bytes per query as the roofline contract defines them for this
-    # path: query row, 8 bytes (key, id) per search probe and per visited entry,
-    # one data row per promoted point, k results.  This engine stores ids apart
-    # from keys, 2 bytes each, and reads keys only where priorities are needed, so
-    # the bytes it has to move for the same work are far fewer: own_layout below.
-    bytes_per_query = 4 * dim + 8 * S + 8 * V + 4 * dim * C + 8 * k
-    bytes_own = 4 * dim + 4 * float(own[2]) + 2 * float(own[0]) + 4 * dim * C + 8 * k + 4 * M * L * C
-    trav_avg_ms = float(np.mean(trav_ms))
-    achieved = bytes_per_query * nq / (trav_avg_ms * 1e-3) / 1e9
-    kernel = "traverse_kernel" if a.traversal == "step" else "traverse_block_kernel"
-    default_run = (a.config == "c2" and cfg == TUNED["c2"] and a.traversal == "auto"
-                   and N == workloads.SHAPES[2]["n"] and nq == workloads.SHAPES[2]["nq"])
-    roofline = dict(bound="hbm", kernel=kernel, achieved=achieved, peak=HBM_PEAK_GBS,
-                    unit="GB/s", frac=achieved / HBM_PEAK_GBS,
-                    traffic=MEASURED_TRAFFIC_C2_DEFAULT if default_run else None,
-                    bytes_per_launch=bytes_per_query * nq, avg_launch_ms=trav_avg_ms,
-                    own_layout_bytes_per_launch=bytes_own * nq,
-                    own_layout_gbs=bytes_own * nq / (trav_avg_ms * 1e-3) / 1e9,
-                    note="achieved prices every visit at the reference's 8 bytes per (key, id) entry; "
-                         "this engine streams 2-byte ids and keeps a partition's slices in the XCD's "
-                         "L2, so achieved can exceed the HBM peak while the measured traffic is far "
-                         "below it: the kernel is bound by vector-ALU issue and memory latency, not "
-                         "by HBM bandwidth")
-    if roofline["traffic"]:
-        roofline["traffic_gbs"] = roofline["traffic"] / (trav_avg_ms * 1e-3) / 1e9
-    build_bytes_proj = 4.0 * N * (dim + I)
+    build_bytes_proj = 4.0 * new_rows * (dim + I)
     build_bytes_sort = 12.0 * N * I
-    build = dict(points_per_s=N / build_wall, wall_ms=build_wall * 1e3,
+    build = dict(points_per_s=new_rows / build_wall, wall_ms=build_wall * 1e3,
                  first_add_wall_ms=build_cold * 1e3,
                  project_ms=proj_t, segsort_ms=sort_t,
                  project_gbs=build_bytes_proj / (proj_t * 1e-3) / 1e9,
                  segsort_gbs=build_bytes_sort / (sort_t * 1e-3) / 1e9,
                  project_frac=build_bytes_proj / (proj_t * 1e-3) / 1e9 / HBM_PEAK_GBS,
                  segsort_frac=build_bytes_sort / (sort_t * 1e-3) / 1e9 / HBM_PEAK_GBS)
+    if per_size is not None:
+        build["note"] = ("last append: %d new rows projected, all %d rows sorted; "
+                         "points_per_s counts the new rows" % (new_rows, N))
+        build["total_points_per_s"] = N / build_wall
 
-    # ---- CPU baseline: the oracle on this box's host cores, bounded sample ----
+    # ---- extras: sweep of num_outer_iterations, blind querying ------------------------
+    outer_sweep = None
+    blind = None
+    if not a.no_extras:
+        if config == "c2":
+            outer_sweep = []
+            say("sweep of num_outer_iterations")
+            for o in (500, 1000, 2000, 5000, 10000, 20000):
+                dci.query(Qd, k, o)
+                torch.cuda.synchronize()
+                t0 = time.perf_counter()
+                for _ in range(2):
+                    oi, _ = dci.query(Qd, k, o, return_int=True)
+                torch.cuda.synchronize()
+                dt = (time.perf_counter() - t0) / 2
+                outer_sweep.append(dict(num_outer_iterations=o, queries_per_s=nq / dt,
+                                        recall_at_k=workloads.recall_at_k(oi[:nrec], truth)))
+            dci.query(Qd, k, outer)
+        if min(10 * k, outer) <= 8192:
+            # no distances: per query the first min(10k, outer) promoted candidates by promoting step
+            nqb = min(nq, legs["blind"])
+            say("blind querying of", nqb, "queries")
+            Qb = Qd[:nqb].contiguous()
+            bids, _ = dci.query(Qb, k, outer, blind=True, return_int=True)
+            torch.cuda.synchronize()
+            reps = min(a.steps, 3)
+            t0 = time.perf_counter()
+            for _ in range(reps):
+                bids, _ = dci.query(Qb, k, outer, blind=True, return_int=True)
+            torch.cuda.synchronize()
+            blind_ms = (time.perf_counter() - t0) * 1e3 / reps
+            nb = min(nqb, nrec)
+            hit = (truth[:nb].unsqueeze(2) == bids[:nb].long().unsqueeze(1)).any(2).float().mean().item()
+            blind = dict(queries_per_s=nqb / (blind_ms * 1e-3), ms_per_step=blind_ms, queries=nqb,
+                         slots_per_query=int(bids.shape[1]), true_neighbours_among_slots=hit)
+
+    # ---- CPU baseline: the oracle on this box's host cores, bounded sample ----------
     cpu = None
     if not a.no_cpu:
         from oracle import dci_oracle as O
+        say("CPU baseline")
         P = dci.directions.numpy()
-        Xn = X.numpy()
-        nqb = min(nq, a.cpu_queries)
+        Xn = X_cpu_sample.numpy()
+        n_cpu = Xn.shape[0]
+        scale = n_cpu / float(N)          # the sample keeps the points per partition
+        bs_cpu = max(1, int(round(cfg["bs"] * scale)))
+        nqb = min(nq, legs["cpu"])
         Qn = Q[:nqb].numpy()
         t0 = time.perf_counter()
-        skeys, sids = O.build_index(P, Xn, cfg["bs"])
+        skeys, sids = O.build_index(P, Xn, bs_cpu)
         t_build = time.perf_counter() - t0
         qproj = O.project(Qn, P)
+        say("CPU index built in %.1f s; querying" % t_build)
         t0 = time.perf_counter()
-        ref = O.query(skeys, sids, Xn, Qn, qproj, M, L, cfg["bs"], cfg["ts"], k, cfg["outer"])
+        ref = O.query(skeys, sids, Xn, Qn, qproj, M, L, bs_cpu, cfg["ts"], k, outer)
         t_query = time.perf_counter() - t0
-        agree = float(np.mean([len(set(x.tolist()) & set(y.tolist())) / k
-                               for x, y in zip(ids[:nqb].cpu().numpy(), ref["ids"])]))
+        agree = None
+        if n_cpu == N:
+            agree = float(np.mean([len(set(x.tolist()) & set(y.tolist())) / k
+                                   for x, y in zip(ids[:nqb].cpu().numpy(), ref["ids"])]))
+        nex = min(nqb, 128)
         t0 = time.perf_counter()
-        Xt, Qt = torch.from_numpy(Xn), torch.from_numpy(Qn[:min(nqb, 128)])
-        torch.cdist(Qt, Xt).topk(k, largest=False)
+        torch.cdist(torch.from_numpy(Qn[:nex]), torch.from_numpy(Xn)).topk(k, largest=False)
         t_exact = time.perf_counter() - t0
-        cpu = dict(value=nqb / t_query, unit="queries/s", cores=O.max_threads(), kind="port",
-                   sample="oracle (CPU restatement of the reference algorithm) on the first %d "
-                          "queries of the same workload, same (bs, ts, outer); build timed on "
-                          "all %d points" % (nqb, N),
-                   build_points_per_s=N / t_build, set_agreement_with_gpu=agree,
-                   exact_cdist_topk_queries_per_s=min(nqb, 128) / t_exact,
+        if n_cpu == N:
+            sample = ("oracle (CPU restatement of the reference algorithm) on the first %d queries of the "
+                      "same workload, same (bs, ts, outer); build timed on all %d points" % (nqb, N))
+        else:
+            sample = ("oracle (CPU restatement of the reference algorithm) on the first %d points and %d "
+                      "queries of the same workload with block_size %d (the same %d points per partition), "
+                      "same (ts, outer); a query's work is proportional to the number of partitions, so "
+                      "value = the measured %.1f queries/s x %d / %d" %
+                      (n_cpu, nqb, bs_cpu, ppb, nqb / t_query, n_cpu, N))
+        cpu = dict(value=nqb / t_query * scale, unit="queries/s", cores=O.max_threads(), kind="port",
+                   sample=sample, measured_queries_per_s_on_sample=nqb / t_query,
+                   sample_points=n_cpu, sample_queries=nqb, seconds=t_query + t_build,
+                   build_points_per_s=n_cpu / t_build, set_agreement_with_gpu=agree,
+                   exact_cdist_topk_queries_per_s=nex / t_exact * scale,
                    host_cpus=os.cpu_count(), torch_threads=torch.get_num_threads())
 
     out = {
         "metric": "queries/sec at recall@10>=0.95, 1Mx128 fp32 k=10; index build points/sec"
-                  if a.config == "c2" else "queries/sec; index build points/sec",
+                  if config == "c2" else "queries/sec; index build points/sec",
         "value": qps, "unit": "queries/s", "n_gpus": 1, "steps": a.steps, "warmup": a.warmup,
         "ms_per_step": ms_per_step, "higher_is_better": True, "scaling": "weak",
         "vs_baseline": None, "dtype": "f32", "data": "synthetic",
-        "config": {"workload": "%s: %d pts x %d fp32, %d queries, m=%d L=%d k=%d" %
-                               (a.config.upper(), N, dim, nq, M, L, k),
+        "config": {"workload": workload_text,
                    "block_size": cfg["bs"], "thread_size": cfg["ts"],
-                   "num_outer_iterations": cfg["outer"]},
-        "recall_at_k": recall, "recall_ok": recall >= 0.95,
-        "build_points_per_s": N / build_wall,
+                   "num_outer_iterations": outer},
+        "recall_at_k": recall, "recall_queries": nrec, "recall_target": target,
+        "recall_ok": None if target is None else recall >= target,
+        "build_points_per_s": new_rows / build_wall,
         "per_query": {"visited": V, "candidates": C, "probes": S, "outer_steps": steps_q,
-                      "algorithmic_bytes": bytes_per_query, "counter_sample_queries": nqc,
-                      "entries_streamed_by_timed_kernel": float(own[0]),
-                      "key_reads_by_timed_kernel": float(own[2])},
-        "kernel_ms": {"traverse": trav_avg_ms, "merge": float(np.mean(merge_ms)),
-                      "query_project": float(np.mean(qproj_ms))},
+                      "contract_bytes": contract_bytes, "counter_sample_queries": nqc,
+                      "entries_streamed_by_timed_kernels": float(own[0]),
+                      "key_reads_by_timed_kernels": float(own[2])},
+        "kernel_ms": {"traverse": trav_ms, "batch_kernel": batch_ms, "dense_kernel": dense_ms,
+                      "merge": tavg[_capi.T_MERGE], "query_project": tavg[_capi.T_QPROJECT]},
         "build": build,
+        "first_call": first_call,
+        "outer_sweep": outer_sweep,
         "blind": blind,
+        "per_size": per_size,
         "roofline": roofline,
         "cpu_baseline": cpu,
     }

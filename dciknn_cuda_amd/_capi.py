@@ -13,10 +13,11 @@ NUM_COUNTERS = 4
 CTR_VISITED, CTR_CANDIDATES, CTR_PROBES, CTR_STEPS = range(4)
 OPT_TRAVERSAL = 0
 OPT_DENSE_MIN_PROMOTIONS = 1
+OPT_FORGET_HINTS = 2
 TRAVERSAL_AUTO, TRAVERSAL_STEP, TRAVERSAL_BATCH, TRAVERSAL_DENSE = 0, 1, 2, 3
 NOALLOC_SCRATCH_BYTES = 32 << 20
-NUM_TIMERS = 5
-T_PROJECT, T_SEGSORT, T_QPROJECT, T_TRAVERSE, T_MERGE = range(5)
+NUM_TIMERS = 7
+T_PROJECT, T_SEGSORT, T_QPROJECT, T_TRAVERSE, T_MERGE, T_BATCH, T_DENSE = range(7)
 
 # name -> (restype, argtypes); one line per declaration in include/dci_hip.h
 _c = ctypes

@@ -516,6 +516,7 @@ static int query_impl(dcih_index* h, int dim, int num_queries, const float* d_qu
         return 0;
     };
 
+    h->ev_valid[DCIH_T_BATCH] = h->ev_valid[DCIH_T_DENSE] = false;
     QueryArgs a;
     a.skeys = h->d_skeys; a.sids = h->d_sids; a.inv = h->d_inv; a.lids = h->d_lids; a.data = h->d_data; a.query = d_query;
     a.mode = h->traversal; a.item_list = nullptr; a.item_count = nullptr; a.dense = nullptr;
@@ -621,12 +622,16 @@ static int query_impl(dcih_index* h, int dim, int num_queries, const float* d_qu
     rc = project(h->d_dirs, I, d_query, num_queries, dim, d_qproj, num_queries, s);
     mark(h, DCIH_T_QPROJECT, 1, s);
     if (rc) return rc;
-    hipEvent_t qev[3] = {h->ev[2 * DCIH_T_TRAVERSE], h->ev[2 * DCIH_T_TRAVERSE + 1],
-                         h->ev[2 * DCIH_T_MERGE + 1]};
-    rc = query(a, s, h->profiling ? qev : nullptr);
+    // events in the order query() records them: traversal start, batch kernel end, dense
+    // kernel end, traversal end, merge end
+    hipEvent_t qev[5] = {h->ev[2 * DCIH_T_TRAVERSE], h->ev[2 * DCIH_T_BATCH + 1], h->ev[2 * DCIH_T_DENSE + 1],
+                         h->ev[2 * DCIH_T_TRAVERSE + 1], h->ev[2 * DCIH_T_MERGE + 1]};
+    bool ran[2] = {false, false};
+    rc = query(a, s, h->profiling ? qev : nullptr, ran);
     if (rc == DCIH_OK && h->profiling) {
-        // the merge starts where the traversal ends
         h->ev_valid[DCIH_T_TRAVERSE] = h->ev_valid[DCIH_T_MERGE] = true;
+        h->ev_valid[DCIH_T_BATCH] = ran[0];
+        h->ev_valid[DCIH_T_DENSE] = ran[1];
     }
     return rc;
 }
@@ -675,6 +680,10 @@ int dcih_set_option(dcih_index* h, int option, int value) {
         h->dense_min_promos = value;
         return DCIH_OK;
     }
+    if (option == DCIH_OPT_FORGET_HINTS) {
+        h->hint_k = h->hint_outer = h->hint_T = h->hint_maxc = 0;     // the next query clears the table
+        return DCIH_OK;
+    }
     return fail(DCIH_EINVAL, "dcih_set_option: unknown option or value");
 }
 
@@ -702,8 +711,12 @@ int dcih_last_timings(dcih_index* h, float* h_ms) {
     for (int t = 0; t < DCIH_NUM_TIMERS; t++) {
         h_ms[t] = -1.0f;
         if (!h->ev_valid[t]) continue;
-        // the merge timer shares its start with the traversal's end event
-        hipEvent_t a = t == DCIH_T_MERGE ? h->ev[2 * DCIH_T_TRAVERSE + 1] : h->ev[2 * t];
+        // timers that start where another one ends: the merge after the traversal, the batch
+        // kernel at the traversal's start, the dense kernel after the batch kernel
+        hipEvent_t a = h->ev[2 * t];
+        if (t == DCIH_T_MERGE) a = h->ev[2 * DCIH_T_TRAVERSE + 1];
+        if (t == DCIH_T_BATCH) a = h->ev[2 * DCIH_T_TRAVERSE];
+        if (t == DCIH_T_DENSE) a = h->ev_valid[DCIH_T_BATCH] ? h->ev[2 * DCIH_T_BATCH + 1] : h->ev[2 * DCIH_T_TRAVERSE];
         hipEvent_t b = h->ev[2 * t + 1];
         DCIH_HIP(hipEventSynchronize(b));
         DCIH_HIP(hipEventElapsedTime(&h_ms[t], a, b));

@@ -139,8 +139,9 @@ int rank_rows(void* ws, int chunk, int rows, int64_t N, int k, bool inf_is_empty
 // (d_dirs), chunk by chunk; ws = I*chunk floats + exhaustive_ws_bytes(N, chunk) bytes.
 int query_dense(const QueryArgs& a, const float* d_dirs, void* ws, int chunk, hipStream_t s);
 
-// ev: null, or three events recorded before the traversal, between traversal
-// and merge, and after the merge.
-int query(const QueryArgs& a, hipStream_t s, hipEvent_t* ev);
+// ev: null, or five events recorded before the traversal, after the batch kernel (if it
+// ran: ran[0]), after the dense kernel (if it ran: ran[1]), between traversal and merge,
+// and after the merge.
+int query(const QueryArgs& a, hipStream_t s, hipEvent_t* ev, bool* ran);
 
 }  // namespace dcih

@@ -359,7 +359,7 @@ size_t query_gscratch_bytes(const QueryArgs& a) {
     return (size_t)traverse_grid(a, y) * (size_t)y.counter_words * 4;
 }
 
-int query(const QueryArgs& a_in, hipStream_t s, hipEvent_t* ev) {
+int query(const QueryArgs& a_in, hipStream_t s, hipEvent_t* ev, bool* ran) {
     QueryArgs a = a_in;
     if (a.nq <= 0) return 0;
     if (a.k > 8192)
@@ -400,10 +400,14 @@ int query(const QueryArgs& a_in, hipStream_t s, hipEvent_t* ev) {
         if (use_block) {
             const int rc = query_block(a, s);
             if (rc) return rc;
+            if (ev) (void)hipEventRecord(ev[1], s);
+            if (ran) ran[0] = true;
         }
         if (a.mode == 3 || a.dense_items) {
             const int rc = query_dense_items(a, s);
             if (rc) return rc;
+            if (ev) (void)hipEventRecord(ev[2], s);
+            if (ran) ran[1] = true;
         }
         // whatever those kernels handed back goes through the step-by-step kernel
         a.item_list = a.redo_items;
@@ -420,11 +424,11 @@ int query(const QueryArgs& a_in, hipStream_t s, hipEvent_t* ev) {
         }
     }
     DCIH_HIP(hipGetLastError());
-    if (ev) (void)hipEventRecord(ev[1], s);
+    if (ev) (void)hipEventRecord(ev[3], s);
     const int cap = merge_cap(a.k);
     hipLaunchKernelGGL(merge_topk_kernel, dim3((unsigned)a.nq), dim3(kMergeThreads),
                        (size_t)cap * sizeof(unsigned long long), s, a, cap);
-    if (ev) (void)hipEventRecord(ev[2], s);
+    if (ev) (void)hipEventRecord(ev[4], s);
     DCIH_HIP(hipGetLastError());
     return 0;
 }

@@ -44,9 +44,11 @@ enum {
     DCIH_T_PROJECT = 0,   /* build: projection of the data            */
     DCIH_T_SEGSORT = 1,   /* build: segmented sort                    */
     DCIH_T_QPROJECT = 2,  /* query: projection of the queries         */
-    DCIH_T_TRAVERSE = 3,  /* query: traversal + distances + top-k     */
+    DCIH_T_TRAVERSE = 3,  /* query: traversal + distances + top-k, all kernels of it */
     DCIH_T_MERGE = 4,     /* query: merge of the per-partition top-k  */
-    DCIH_NUM_TIMERS = 5
+    DCIH_T_BATCH = 5,     /* query: the batch kernel's share of DCIH_T_TRAVERSE (all its launches) */
+    DCIH_T_DENSE = 6,     /* query: the dense kernel's share of DCIH_T_TRAVERSE */
+    DCIH_NUM_TIMERS = 7
 };
 
 /*
@@ -64,8 +66,11 @@ enum {
  * DCIH_CTR_PROBES their own key reads.  DCIH_OPT_DENSE_MIN_PROMOTIONS: under
  * automatic choice, the number of promotions per (query, partition) from which
  * an item goes to the dense kernel (default 384; 0 = never).
+ * DCIH_OPT_FORGET_HINTS (value ignored): drops what earlier queries taught the
+ * handle about where traversals stop (used only to size the batch kernel's
+ * epochs, never visible in results), so that the next call runs like a first one.
  */
-enum { DCIH_OPT_TRAVERSAL = 0, DCIH_OPT_DENSE_MIN_PROMOTIONS = 1 };
+enum { DCIH_OPT_TRAVERSAL = 0, DCIH_OPT_DENSE_MIN_PROMOTIONS = 1, DCIH_OPT_FORGET_HINTS = 2 };
 
 /* Message for the last failing call on this thread ("" if none). */
 const char* dcih_last_error(void);
