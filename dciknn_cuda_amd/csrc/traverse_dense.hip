@@ -265,37 +265,45 @@ __global__ __launch_bounds__(kDT, 2) void traverse_dense_kernel(QueryArgs a, Den
             __syncthreads();
 
             // ---- every point: the latest of the steps of its L windows ------------------
-            // (sixteen points per thread at a time, so that as many reads of the inverse
-            //  permutation are in flight)
-            constexpr int kP = 16;
+            // (sixteen points per thread at a time and four simple indices at once, so that
+            //  sixty-four reads of the inverse permutation are in flight per lane: the phase is
+            //  a chain of memory round trips and this makes it a short one)
+            constexpr int kP = 16, kH = 4;
             const uint16_t* invm = a.inv + (int64_t)m * a.L * a.N + off;
             for (int c0 = 0; c0 < n; c0 += kDT * kP) {
                 int tmax[kP];
                 uint32_t l0mask = 0;
 #pragma unroll
                 for (int u = 0; u < kP; u++) tmax[u] = -1;
-                for (int h = 0; h < a.L; h++) {
-                    const int i = m * a.L + h;
-                    const int p = s_p[i], sl = s_startL[i], sr = s_startR[i];
-                    const uint16_t* invh = invm + (int64_t)h * a.N;
-                    int posv[kP];
+                for (int h0 = 0; h0 < a.L; h0 += kH) {
+                    int posv[kH][kP];
 #pragma unroll
-                    for (int u = 0; u < kP; u++) posv[u] = (int)invh[min(c0 + u * kDT + tid, n - 1)];
+                    for (int hh = 0; hh < kH; hh++) {
+                        const uint16_t* invh = invm + (int64_t)min(h0 + hh, a.L - 1) * a.N;
 #pragma unroll
-                    for (int u = 0; u < kP; u++) {
-                        const int pos = posv[u];
-                        int idx, t;
-                        if (pos > p) {
-                            const int d = pos - (p + 1), j = div_T(d);
-                            t = d - j * T; idx = sr + j;
-                        } else {
-                            const int d = p - pos, j = div_T(d);
-                            t = pos - (p - T + 1 - j * T); idx = sl + j;
-                        }
-                        const int r = (int)rank16[idx];
-                        if (r > tmax[u]) {
-                            tmax[u] = r;
-                            l0mask = (l0mask & ~(1u << u)) | ((t == 0 ? 1u : 0u) << u);
+                        for (int u = 0; u < kP; u++) posv[hh][u] = (int)invh[min(c0 + u * kDT + tid, n - 1)];
+                    }
+#pragma unroll
+                    for (int hh = 0; hh < kH; hh++) {
+                        if (h0 + hh >= a.L) break;
+                        const int i = m * a.L + h0 + hh;
+                        const int p = s_p[i], sl = s_startL[i], sr = s_startR[i];
+#pragma unroll
+                        for (int u = 0; u < kP; u++) {
+                            const int pos = posv[hh][u];
+                            int idx, t;
+                            if (pos > p) {
+                                const int d = pos - (p + 1), j = div_T(d);
+                                t = d - j * T; idx = sr + j;
+                            } else {
+                                const int d = p - pos, j = div_T(d);
+                                t = pos - (p - T + 1 - j * T); idx = sl + j;
+                            }
+                            const int r = (int)rank16[idx];
+                            if (r > tmax[u]) {
+                                tmax[u] = r;
+                                l0mask = (l0mask & ~(1u << u)) | ((t == 0 ? 1u : 0u) << u);
+                            }
                         }
                     }
                 }
@@ -430,7 +438,8 @@ __global__ __launch_bounds__(kDT, 2) void traverse_dense_kernel(QueryArgs a, Den
                         for (int r = 0; r < R; r++) rows[r] = a.data + (off + pts[r]) * a.dim;
                         float d[R];
                         const float* const (&crows)[R] = rows;
-                        wave_row_dists<R>(crows, s_q, a.dim, vec4, d);
+                        if (R > 2) wave_row_dists_deep<R, 2>(crows, s_q, a.dim, d);      // (only chosen for aligned rows)
+                        else wave_row_dists<R>(crows, s_q, a.dim, vec4, d);
 #pragma unroll
                         for (int r = 0; r < R; r++)
                             e[r] = ((unsigned long long)__builtin_bit_cast(uint32_t, d[r]) << 32) | (uint32_t)(off + pts[r]);
@@ -494,9 +503,12 @@ __global__ __launch_bounds__(kDT, 2) void traverse_dense_kernel(QueryArgs a, Den
         };
         {
             using std::integral_constant;
-            if (vec4 && !a.blind && a.dim <= 64 && y.quota >= 16) run_rounds(integral_constant<int, 16>{}, integral_constant<int, 4>{});
+            if (vec4 && !a.blind && a.dim <= 64 && y.quota >= 32) run_rounds(integral_constant<int, 16>{}, integral_constant<int, 8>{});
+            else if (vec4 && !a.blind && a.dim <= 64 && y.quota >= 16) run_rounds(integral_constant<int, 16>{}, integral_constant<int, 4>{});
             else if (vec4 && !a.blind && a.dim <= 64) run_rounds(integral_constant<int, 16>{}, integral_constant<int, 2>{});
+            else if (vec4 && !a.blind && a.dim <= 128 && y.quota >= 16) run_rounds(integral_constant<int, 32>{}, integral_constant<int, 8>{});
             else if (vec4 && !a.blind && a.dim <= 128) run_rounds(integral_constant<int, 32>{}, integral_constant<int, 4>{});
+            else if (vec4 && !a.blind && a.dim >= 512 && y.quota >= 8) run_rounds(integral_constant<int, 64>{}, integral_constant<int, 8>{});
             else run_rounds(integral_constant<int, 64>{}, integral_constant<int, 2>{});
         }
         if (lane == 0) atomicAdd(&misc[dCand], ncand);
