@@ -46,15 +46,18 @@ enum DMisc {   // 32-bit scalars shared by the workgroup
 struct DenseLayout {
     int ipt;          // windows per thread the sort holds (cap = 256 * ipt per composite)
     int off_idx;      // per simple index: p, qp, left start, right start   (4 * I words)
-    int off_seg;      // per composite: 2L + 1 segment starts, 2L stream numbers
+    int off_seg;      // per composite: 2L + 1 segment starts, 2L stream numbers, 2L table places of window 0
     int off_q;        // query row
     int off_time;     // uint16 per point: step << 1 | lane-0 flag
     int off_sort;     // k best + pending candidates, 64-bit words
     int off_stage;    // radix staging; later the rank table, then the step histogram
     int off_misc, off_wlist;
     int sort_cap, quota;
+    int tiles;        // 1: rows of at most 128 elements, 16-byte aligned, distances wanted: whole batches of 64 rows
     size_t lds_bytes;
 };
+
+constexpr int kWlist = 2 * kWave;        // candidates a wavefront keeps listed
 
 int dense_ipt_for(int64_t windows) {
     for (int ipt : {9, 17, 25, 33})
@@ -73,20 +76,46 @@ DenseLayout make_dense_layout(const QueryArgs& a) {
     int o = dMiscWords * 4 + 64 * 4;      // scalars, then scratch of the block scans
     y.off_misc = 0;
     y.off_idx = o;      o += 4 * I * 4;
-    y.off_seg = o;      o += (4 * a.L + 2) * 4;
+    y.off_seg = o;      o += (6 * a.L + 2) * 4;
     y.off_q = o;        o += ((a.dim + 3) & ~3) * 4;
     y.off_time = o;     o += (int)(((a.ppb + 1) & ~(int64_t)1) * 2);
     o = (o + 15) & ~15;
     // k best plus room for candidates that beat the current k-th: four wavefronts fill
     // a quota each between two merges
+    // (batches of 64 rows: room for one whole batch beyond what a wavefront may hold already)
+    y.tiles = (!a.blind && a.dim <= 128 && (a.dim & 3) == 0 &&
+               (reinterpret_cast<uintptr_t>(a.data) & 15) == 0) ? 1 : 0;
     y.sort_cap = 64;
-    while (y.sort_cap < a.kcap + 4 * 8) y.sort_cap <<= 1;
+    while (y.sort_cap < a.kcap + 4 * (y.tiles ? 96 : 8)) y.sort_cap <<= 1;
     y.quota = (y.sort_cap - a.kcap) / kDWaves;
     y.off_sort = o;     o += y.sort_cap * 8;
-    y.off_wlist = o;    o += kDWaves * kWave * 2;
+    y.off_wlist = o;    o += kDWaves * kWlist * 2;
     y.off_stage = o;    o += (y.ipt + 8) * kDT * 4;      // staging words, then the digit counters
     y.lds_bytes = (size_t)o;
     return y;
+}
+
+// Sums of N rows' lane values over a group of N lanes at once: on entry lane s of the group
+// holds v[r] = its share of row r; on return it holds the total of row s.  Each level pairs
+// the lanes s and s ^ H and halves the rows a lane carries, adding exactly the operands the
+// butterfly  v += shfl_xor(v, H)  of wave_sum adds for that row, in the same order of levels,
+// so every total has the bits wave_row_dists gives (N - 1 exchanges for N rows, not N log N).
+template <int N>
+__device__ inline float group_row_sums(float (&v)[N], int s) {
+    if constexpr (N == 1) {
+        return v[0];
+    } else {
+        constexpr int H = N / 2;
+        const bool upper = (s & H) != 0;
+        float nv[H];
+#pragma unroll
+        for (int i = 0; i < H; i++) {
+            const float send = upper ? v[i] : v[i + H];
+            const float keep = upper ? v[i + H] : v[i];
+            nv[i] = keep + __shfl_xor(send, H, kWave);
+        }
+        return group_row_sums<H>(nv, s);
+    }
 }
 
 template <int IPT>
@@ -96,8 +125,11 @@ __global__ __launch_bounds__(kDT, 2) void traverse_dense_kernel(QueryArgs a, Den
     uint32_t* scan_tmp = misc + dMiscWords;                           // 64 words
     int* s_p = reinterpret_cast<int*>(smem + y.off_idx);
     float* s_qp = reinterpret_cast<float*>(s_p + a.M * a.L);
-    int* s_startL = reinterpret_cast<int*>(s_qp + a.M * a.L);         // layout index of a stream's window 0
-    int* s_startR = s_startL + a.M * a.L;
+    // per simple index: where its windows start in the step table (there they lie in the order
+    // of the positions they cover), and the shift that makes (position + shift) / T a window's
+    // place among them
+    int* s_tabbase = reinterpret_cast<int*>(s_qp + a.M * a.L);
+    int* s_shift = s_tabbase + a.M * a.L;
     int* s_seg = reinterpret_cast<int*>(smem + y.off_seg);            // 2L + 1 segment starts (layout order)
     int* s_segstream = s_seg + 2 * a.L + 1;                           // stream (2h + side) of a segment
     float* s_q = reinterpret_cast<float*>(smem + y.off_q);
@@ -105,7 +137,8 @@ __global__ __launch_bounds__(kDT, 2) void traverse_dense_kernel(QueryArgs a, Den
     unsigned long long* sortbuf = reinterpret_cast<unsigned long long*>(smem + y.off_sort);
     uint32_t* stage = reinterpret_cast<uint32_t*>(smem + y.off_stage);
     uint16_t* rank16 = reinterpret_cast<uint16_t*>(stage);
-    uint16_t* s_wlist = reinterpret_cast<uint16_t*>(smem + y.off_wlist);   // per wavefront: 64 candidates
+    uint16_t* s_wlist = reinterpret_cast<uint16_t*>(smem + y.off_wlist);   // per wavefront: kWlist candidates
+    int* s_segw = s_segstream + 2 * a.L;                              // table place of a segment's window 0
 
     const int tid = threadIdx.x;
     const int lane = tid & (kWave - 1);
@@ -185,12 +218,19 @@ __global__ __launch_bounds__(kDT, 2) void traverse_dense_kernel(QueryArgs a, Den
                     const int i = m * a.L + h, p = s_p[i];
                     const int nl = stream_windows(n, T, p, 0), nr = stream_windows(n, T, p, 1);
                     const bool corner = p == n - 1 && T >= 2;
+                    // In the table the index's windows lie by the positions they cover: left
+                    // window j at place nl - 1 - j, right window j at nl + j; a position pos
+                    // belongs to the window at place (pos + nl * T - p - 1) / T and is its first
+                    // lane where that division leaves no remainder.
+                    s_tabbase[i] = at;
+                    s_shift[i] = nl * T - p - 1;
+                    const int w_left = at + nl - 1, w_right = at + nl;
                     if (corner) {
-                        s_seg[2 * h] = at; s_segstream[2 * h] = 2 * h + 1; s_startR[i] = at; at += nr;
-                        s_seg[2 * h + 1] = at; s_segstream[2 * h + 1] = 2 * h; s_startL[i] = at; at += nl;
+                        s_seg[2 * h] = at; s_segstream[2 * h] = 2 * h + 1; s_segw[2 * h] = w_right; at += nr;
+                        s_seg[2 * h + 1] = at; s_segstream[2 * h + 1] = 2 * h; s_segw[2 * h + 1] = w_left; at += nl;
                     } else {
-                        s_seg[2 * h] = at; s_segstream[2 * h] = 2 * h; s_startL[i] = at; at += nl;
-                        s_seg[2 * h + 1] = at; s_segstream[2 * h + 1] = 2 * h + 1; s_startR[i] = at; at += nr;
+                        s_seg[2 * h] = at; s_segstream[2 * h] = 2 * h; s_segw[2 * h] = w_left; at += nl;
+                        s_seg[2 * h + 1] = at; s_segstream[2 * h + 1] = 2 * h + 1; s_segw[2 * h + 1] = w_right; at += nr;
                     }
                 }
                 s_seg[2 * a.L] = at;
@@ -212,6 +252,7 @@ __global__ __launch_bounds__(kDT, 2) void traverse_dense_kernel(QueryArgs a, Den
                 int seg_end = s_seg[seg + 1];
                 int sidx = s_segstream[seg];
                 int seg_at = s_seg[seg];
+                int seg_w = s_segw[seg];
                 // (offsets from the composite's first slice; all reads are issued before any is used)
                 const float* kbase = a.skeys + (int64_t)m * a.L * a.N + off;
                 uint32_t koff[IPT];
@@ -221,12 +262,13 @@ __global__ __launch_bounds__(kDT, 2) void traverse_dense_kernel(QueryArgs a, Den
                     const int idx = first + r;
                     while (idx >= seg_end && seg < 2 * a.L - 1) {
                         seg++;
-                        seg_end = s_seg[seg + 1]; sidx = s_segstream[seg]; seg_at = s_seg[seg];
+                        seg_end = s_seg[seg + 1]; sidx = s_segstream[seg]; seg_at = s_seg[seg]; seg_w = s_segw[seg];
                     }
                     const int h = sidx >> 1, p = s_p[m * a.L + h], j = idx - seg_at;
                     const int pos = (sidx & 1) ? min(p + 1 + j * T, n - 1) : max(p - T + 1 - j * T, 0);
                     koff[r] = (uint32_t)h * (uint32_t)a.N + (uint32_t)(idx < W ? pos : 0);
                     qv[r] = s_qp[m * a.L + h];
+                    rp[r] = (uint32_t)(idx < W ? ((sidx & 1) ? seg_w + j : seg_w - j) : 0);    // the sort's payload: the window's place in the table
                 }
                 float kv[IPT];
 #pragma unroll
@@ -237,7 +279,6 @@ __global__ __launch_bounds__(kDT, 2) void traverse_dense_kernel(QueryArgs a, Den
                     const int idx = first + r;
                     const uint32_t bits = __builtin_bit_cast(uint32_t, fabsf(kv[r] - qv[r]));
                     k[r] = idx < W ? bits : 0xffffffffu;      // pads sort last and stay last
-                    rp[r] = (uint32_t)idx;
                     vor |= idx < W ? bits : 0u;
                     vand &= idx < W ? bits : 0xffffffffu;
                 }
@@ -256,11 +297,12 @@ __global__ __launch_bounds__(kDT, 2) void traverse_dense_kernel(QueryArgs a, Den
             lds_radix_passes<kDT, IPT>(k, rp, stage, stage + IPT * kDT, scan_tmp, varying);
             __syncthreads();
             phase(2);
-            // the step of every window: its place in the sorted order
+            // the step of every window: its place in the sorted order (the first W sorted items
+            // are the windows), stored doubled so that the lane-0 flag fits beside it
 #pragma unroll
             for (int r = 0; r < IPT; r++) {
-                const uint32_t idx = rp[r] & 0xffffu;
-                if (idx < (uint32_t)W) rank16[idx] = (uint16_t)(tid * IPT + r);
+                const int sp = tid * IPT + r;
+                if (sp < W) rank16[rp[r] & 0xffffu] = (uint16_t)(sp << 1);
             }
             __syncthreads();
 
@@ -271,10 +313,9 @@ __global__ __launch_bounds__(kDT, 2) void traverse_dense_kernel(QueryArgs a, Den
             constexpr int kP = 16, kH = 4;
             const uint16_t* invm = a.inv + (int64_t)m * a.L * a.N + off;
             for (int c0 = 0; c0 < n; c0 += kDT * kP) {
-                int tmax[kP];
-                uint32_t l0mask = 0;
+                uint32_t best[kP];         // step << 1 | lane-0 flag of the latest window so far
 #pragma unroll
-                for (int u = 0; u < kP; u++) tmax[u] = -1;
+                for (int u = 0; u < kP; u++) best[u] = 0u;
                 for (int h0 = 0; h0 < a.L; h0 += kH) {
                     int posv[kH][kP];
 #pragma unroll
@@ -287,23 +328,13 @@ __global__ __launch_bounds__(kDT, 2) void traverse_dense_kernel(QueryArgs a, Den
                     for (int hh = 0; hh < kH; hh++) {
                         if (h0 + hh >= a.L) break;
                         const int i = m * a.L + h0 + hh;
-                        const int p = s_p[i], sl = s_startL[i], sr = s_startR[i];
+                        const int shift = s_shift[i];
+                        const uint16_t* tab = rank16 + s_tabbase[i];
 #pragma unroll
                         for (int u = 0; u < kP; u++) {
-                            const int pos = posv[hh][u];
-                            int idx, t;
-                            if (pos > p) {
-                                const int d = pos - (p + 1), j = div_T(d);
-                                t = d - j * T; idx = sr + j;
-                            } else {
-                                const int d = p - pos, j = div_T(d);
-                                t = pos - (p - T + 1 - j * T); idx = sl + j;
-                            }
-                            const int r = (int)rank16[idx];
-                            if (r > tmax[u]) {
-                                tmax[u] = r;
-                                l0mask = (l0mask & ~(1u << u)) | ((t == 0 ? 1u : 0u) << u);
-                            }
+                            const int x = posv[hh][u] + shift, w = div_T(x);
+                            const uint32_t v = (uint32_t)tab[w] | (x - w * T == 0 ? 1u : 0u);
+                            best[u] = max(best[u], v);      // (steps differ from window to window)
                         }
                     }
                 }
@@ -312,7 +343,7 @@ __global__ __launch_bounds__(kDT, 2) void traverse_dense_kernel(QueryArgs a, Den
                     const int pt = c0 + u * kDT + tid;
                     if (pt < n) {
                         const uint32_t old = s_time[pt];      // ties: the earlier composite stays
-                        if ((uint32_t)tmax[u] < (old >> 1)) s_time[pt] = (uint16_t)((tmax[u] << 1) | ((l0mask >> u) & 1u));
+                        if ((best[u] >> 1) < (old >> 1)) s_time[pt] = (uint16_t)best[u];
                     }
                 }
             }
@@ -389,10 +420,33 @@ __global__ __launch_bounds__(kDT, 2) void traverse_dense_kernel(QueryArgs a, Den
         const int chunk = (n + kDWaves - 1) / kDWaves;
         int at = wave * chunk;                              // next point of this wavefront (wave-uniform)
         const int at_end = min(n, at + chunk);
-        uint16_t* wl = s_wlist + wave * kWave;              // this wavefront's candidates among the 64 points loaded last
+        uint16_t* wl = s_wlist + wave * kWlist;             // this wavefront's candidates, listed 64 points at a time
         int list_len = 0, list_pos = 0;
         uint32_t ncand = 0;
         int topn = 0;
+        // end of a round: the wavefronts' pending candidates are merged into the k best;
+        // returns whether any wavefront has points left
+        auto merge_round = [&](int mine, unsigned long long* my_slots) -> bool {
+            for (int j = mine + lane; j < y.quota; j += kWave) my_slots[j] = ~0ull;
+            const bool more = list_pos < list_len || at < at_end;
+            if (lane == 0) {
+                scan_tmp[8 + wave] = (uint32_t)mine;
+                scan_tmp[16 + wave] = more ? 1u : 0u;
+            }
+            // (slots between the k best held so far and the first wavefront's share)
+            for (int j = topn + tid; j < a.kcap; j += kDT) sortbuf[j] = ~0ull;
+            for (int j = a.kcap + kDWaves * y.quota + tid; j < y.sort_cap; j += kDT) sortbuf[j] = ~0ull;
+            __syncthreads();
+            int added = 0, any_more = 0;
+            for (int w2 = 0; w2 < kDWaves; w2++) { added += (int)scan_tmp[8 + w2]; any_more |= (int)scan_tmp[16 + w2]; }
+            if (added > 0) {
+                bitonic_sort_u64(sortbuf, y.sort_cap);
+                topn = min(a.kcap, topn + added);
+            } else {
+                __syncthreads();
+            }
+            return any_more != 0;
+        };
         auto run_rounds = [&](auto gtag, auto rtag) {
             constexpr int GL = decltype(gtag)::value;       // lanes per row
             constexpr int R = decltype(rtag)::value;        // rows per lane group in flight
@@ -432,7 +486,7 @@ __global__ __launch_bounds__(kDT, 2) void traverse_dense_kernel(QueryArgs a, Den
 #pragma unroll
                         for (int r = 0; r < R; r++)
                             e[r] = ((unsigned long long)(s_time[pts[r]] >> 1) << 32) | (uint32_t)(off + pts[r]);
-                    } else if (GL == kWave) {
+                    } else {
                         const float* rows[R];
 #pragma unroll
                         for (int r = 0; r < R; r++) rows[r] = a.data + (off + pts[r]) * a.dim;
@@ -443,33 +497,6 @@ __global__ __launch_bounds__(kDT, 2) void traverse_dense_kernel(QueryArgs a, Den
 #pragma unroll
                         for (int r = 0; r < R; r++)
                             e[r] = ((unsigned long long)__builtin_bit_cast(uint32_t, d[r]) << 32) | (uint32_t)(off + pts[r]);
-                    } else {
-                        typedef float v4f __attribute__((ext_vector_type(4)));
-                        float acc[R];
-                        const int j = sl * 4;
-                        v4f x[R];
-#pragma unroll
-                        for (int r = 0; r < R; r++) {
-                            acc[r] = 0.f;
-                            if (j < a.dim) x[r] = *reinterpret_cast<const v4f*>(a.data + (off + pts[r]) * a.dim + j);
-                        }
-                        if (j < a.dim) {
-                            const float q0 = s_q[j], q1 = s_q[j + 1], q2 = s_q[j + 2], q3 = s_q[j + 3];
-#pragma unroll
-                            for (int r = 0; r < R; r++) {
-                                float dd = x[r].x - q0; acc[r] = __builtin_fmaf(dd, dd, acc[r]);
-                                dd = x[r].y - q1; acc[r] = __builtin_fmaf(dd, dd, acc[r]);
-                                dd = x[r].z - q2; acc[r] = __builtin_fmaf(dd, dd, acc[r]);
-                                dd = x[r].w - q3; acc[r] = __builtin_fmaf(dd, dd, acc[r]);
-                            }
-                        }
-#pragma unroll
-                        for (int r = 0; r < R; r++) {
-                            float v = acc[r];
-#pragma unroll
-                            for (int o = GL / 2; o > 0; o >>= 1) v += __shfl_xor(v, o, kWave);
-                            e[r] = ((unsigned long long)__builtin_bit_cast(uint32_t, sqrtf(v)) << 32) | (uint32_t)(off + pts[r]);
-                        }
                     }
 #pragma unroll
                     for (int r = 0; r < R; r++) {
@@ -480,34 +507,89 @@ __global__ __launch_bounds__(kDT, 2) void traverse_dense_kernel(QueryArgs a, Den
                     }
                     list_pos += RB;
                 }
-                for (int j = mine + lane; j < y.quota; j += kWave) my_slots[j] = ~0ull;
-                const bool more = list_pos < list_len || at < at_end;
-                if (lane == 0) {
-                    scan_tmp[8 + wave] = (uint32_t)mine;
-                    scan_tmp[16 + wave] = more ? 1u : 0u;
+                if (!merge_round(mine, my_slots)) break;
+            }
+        };
+        // Rows of at most 4 * GL elements: a batch is 64 candidates, GL lanes read a row (16
+        // bytes each) and every lane group takes GL rows, eight loads in flight per lane; the
+        // GL partial sums a lane ends up with are reduced for all its rows together, which
+        // leaves lane c of the wavefront with the distance of candidate c: one comparison, one
+        // ballot and one store per batch instead of one per row.
+        auto run_tiles = [&](auto gtag) {
+            typedef float v4f __attribute__((ext_vector_type(4)));
+            constexpr int GL = decltype(gtag)::value;
+            const int grp = lane / GL, sl = lane & (GL - 1);
+            const int j = sl * 4;
+            const bool has = j < a.dim;
+            float q0 = 0.f, q1 = 0.f, q2 = 0.f, q3 = 0.f;
+            if (has) { q0 = s_q[j]; q1 = s_q[j + 1]; q2 = s_q[j + 2]; q3 = s_q[j + 3]; }
+            const float* base = a.data + off * a.dim + (has ? j : 0);
+            for (;;) {
+                unsigned long long kth = ~0ull;
+                if (topn >= a.kcap) kth = sortbuf[a.kcap - 1];
+                int mine = 0;
+                unsigned long long* my_slots = sortbuf + a.kcap + wave * y.quota;
+                for (;;) {
+                    // list at least a whole batch, while points are left
+                    while (list_len - list_pos < kWave && at < at_end) {
+                        if (list_pos > 0) {      // what is left moves to the front (one wavefront: its LDS operations keep their order)
+                            const int rest = list_len - list_pos;
+                            const uint16_t v = lane < rest ? wl[list_pos + lane] : (uint16_t)0;
+                            if (lane < rest) wl[lane] = v;
+                            list_len = rest;
+                            list_pos = 0;
+                        }
+                        const int pt = at + lane;
+                        const uint32_t v = pt < at_end ? (uint32_t)s_time[pt] : 0xffffu;
+                        const bool is_cand = (v >> 1) <= t_lim;
+                        const unsigned long long m = __ballot(is_cand);
+                        if (is_cand) wl[list_len + __popcll(m & ((1ull << lane) - 1ull))] = (uint16_t)pt;
+                        list_len += __popcll(m);
+                        at += kWave;
+                        ncand += (uint32_t)__popcll(m);
+                    }
+                    const int nb = min(kWave, list_len - list_pos);
+                    if (nb <= 0) break;
+                    if (mine + kWave > y.quota) break;      // no room for a whole batch: merge first
+                    const uint16_t* cur = wl + list_pos;
+                    float acc[GL];
+#pragma unroll
+                    for (int r0 = 0; r0 < GL; r0 += 8) {
+                        v4f x[8];
+#pragma unroll
+                        for (int r = 0; r < 8; r++) {
+                            // (lanes beyond the row's end read its head and add nothing: a load
+                            //  under a condition would wait for the loads before it)
+                            const int pt = (int)cur[min(grp * GL + r0 + r, nb - 1)];
+                            x[r] = *reinterpret_cast<const v4f*>(base + pt * a.dim);
+                        }
+#pragma unroll
+                        for (int r = 0; r < 8; r++) {
+                            float s2 = 0.f;
+                            float dd = x[r].x - q0; s2 = __builtin_fmaf(dd, dd, s2);
+                            dd = x[r].y - q1; s2 = __builtin_fmaf(dd, dd, s2);
+                            dd = x[r].z - q2; s2 = __builtin_fmaf(dd, dd, s2);
+                            dd = x[r].w - q3; s2 = __builtin_fmaf(dd, dd, s2);
+                            acc[r0 + r] = has ? s2 : 0.f;
+                        }
+                    }
+                    const float total = group_row_sums<GL>(acc, sl);      // of candidate grp * GL + sl = lane
+                    const int mypt = (int)cur[min(lane, nb - 1)];
+                    const unsigned long long e =
+                        ((unsigned long long)__builtin_bit_cast(uint32_t, sqrtf(total)) << 32) | (uint32_t)(off + mypt);
+                    const bool keep = lane < nb && e < kth;
+                    const unsigned long long m = __ballot(keep);
+                    if (keep) my_slots[mine + __popcll(m & ((1ull << lane) - 1ull))] = e;
+                    mine += __popcll(m);
+                    list_pos += nb;
                 }
-                // (slots between the k best held so far and the first wavefront's share)
-                for (int j = topn + tid; j < a.kcap; j += kDT) sortbuf[j] = ~0ull;
-                for (int j = a.kcap + kDWaves * y.quota + tid; j < y.sort_cap; j += kDT) sortbuf[j] = ~0ull;
-                __syncthreads();
-                int added = 0, any_more = 0;
-                for (int w2 = 0; w2 < kDWaves; w2++) { added += (int)scan_tmp[8 + w2]; any_more |= (int)scan_tmp[16 + w2]; }
-                if (added > 0) {
-                    bitonic_sort_u64(sortbuf, y.sort_cap);
-                    topn = min(a.kcap, topn + added);
-                } else {
-                    __syncthreads();
-                }
-                if (!any_more) break;
+                if (!merge_round(mine, my_slots)) break;
             }
         };
         {
             using std::integral_constant;
-            if (vec4 && !a.blind && a.dim <= 64 && y.quota >= 32) run_rounds(integral_constant<int, 16>{}, integral_constant<int, 8>{});
-            else if (vec4 && !a.blind && a.dim <= 64 && y.quota >= 16) run_rounds(integral_constant<int, 16>{}, integral_constant<int, 4>{});
-            else if (vec4 && !a.blind && a.dim <= 64) run_rounds(integral_constant<int, 16>{}, integral_constant<int, 2>{});
-            else if (vec4 && !a.blind && a.dim <= 128 && y.quota >= 16) run_rounds(integral_constant<int, 32>{}, integral_constant<int, 8>{});
-            else if (vec4 && !a.blind && a.dim <= 128) run_rounds(integral_constant<int, 32>{}, integral_constant<int, 4>{});
+            if (y.tiles && vec4 && a.dim <= 64 && y.quota >= kWave) run_tiles(integral_constant<int, 16>{});
+            else if (y.tiles && vec4 && a.dim <= 128 && y.quota >= kWave) run_tiles(integral_constant<int, 32>{});
             else if (vec4 && !a.blind && a.dim >= 512 && y.quota >= 8) run_rounds(integral_constant<int, 64>{}, integral_constant<int, 8>{});
             else run_rounds(integral_constant<int, 64>{}, integral_constant<int, 2>{});
         }
@@ -548,7 +630,7 @@ bool dense_traversal_supported(const QueryArgs& a, size_t* lds_bytes) {
     if (!a.inv || a.ppb > 32766 || a.T < 1) return false;
     if (a.M > 64 || a.L > 64 || a.kcap > 512 || (int64_t)a.L * a.N >= 0x7fffffffLL) return false;
     if (dense_ipt_for(dense_max_windows(a)) == 0) return false;
-    if (dense_max_windows(a) >= 0x7fff) return false;
+    if (dense_max_windows(a) >= 0x7fff || a.ppb + (int64_t)a.T >= 65536) return false;
     if (a.xcds < 1 || a.xcds > 32 || (int64_t)a.nq * (a.B + a.xcds) >= 0x7fffffffLL) return false;
     const DenseLayout y = make_dense_layout(a);
     if (lds_bytes) *lds_bytes = y.lds_bytes;
