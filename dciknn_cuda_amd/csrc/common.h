@@ -207,6 +207,70 @@ __device__ inline void bitonic_sort_u64(unsigned long long* s, int n) {
     }
     __syncthreads();
 }
+
+// The same sort for n = 256 * E words by a workgroup of exactly 256 threads, E a power of
+// two: every thread keeps E consecutive words in registers, exchanges within a thread and
+// within a wavefront need neither LDS nor a barrier, and only the steps whose partners lie in
+// another wavefront (two or three of them in all) go through `s`.
+template <int E>
+__device__ inline void bitonic_sort_u64_regs(unsigned long long* s) {
+    constexpr int n = 256 * E;
+    const int tid = (int)threadIdx.x;
+    unsigned long long v[E];
+    __syncthreads();
+#pragma unroll
+    for (int i = 0; i < E; i++) v[i] = s[tid * E + i];
+#pragma unroll
+    for (int size = 2; size <= n; size <<= 1) {
+#pragma unroll
+        for (int stride = size >> 1; stride > 0; stride >>= 1) {
+            if (stride >= kWave * E) {
+                __syncthreads();
+#pragma unroll
+                for (int i = 0; i < E; i++) s[tid * E + i] = v[i];
+                __syncthreads();
+#pragma unroll
+                for (int i = 0; i < E; i++) {
+                    const int e = tid * E + i;
+                    const unsigned long long o = s[e ^ stride];
+                    const bool keep_min = ((e & stride) == 0) == ((e & size) == 0);
+                    v[i] = keep_min ? (v[i] < o ? v[i] : o) : (v[i] > o ? v[i] : o);
+                }
+            } else if (stride >= E) {
+#pragma unroll
+                for (int i = 0; i < E; i++) {
+                    const int e = tid * E + i;
+                    const unsigned long long o = __shfl_xor(v[i], stride / E, kWave);
+                    const bool keep_min = ((e & stride) == 0) == ((e & size) == 0);
+                    v[i] = keep_min ? (v[i] < o ? v[i] : o) : (v[i] > o ? v[i] : o);
+                }
+            } else {
+#pragma unroll
+                for (int i = 0; i < E; i++) {
+                    if ((i & stride) == 0) {
+                        const int e = tid * E + i;
+                        const bool up = (e & size) == 0;
+                        const unsigned long long x = v[i], y = v[i | stride];
+                        const bool swap = (x > y) == up;
+                        v[i] = swap ? y : x;
+                        v[i | stride] = swap ? x : y;
+                    }
+                }
+            }
+        }
+    }
+    __syncthreads();
+#pragma unroll
+    for (int i = 0; i < E; i++) s[tid * E + i] = v[i];
+    __syncthreads();
+}
+// n words by 256 threads: the register variant where it applies.
+__device__ inline void bitonic_sort_u64_by256(unsigned long long* s, int n) {
+    if (n == 256) bitonic_sort_u64_regs<1>(s);
+    else if (n == 512) bitonic_sort_u64_regs<2>(s);
+    else if (n == 1024) bitonic_sort_u64_regs<4>(s);
+    else bitonic_sort_u64(s, n);
+}
 #endif
 
 }  // namespace dcih

@@ -440,7 +440,7 @@ __global__ __launch_bounds__(kDT, 2) void traverse_dense_kernel(QueryArgs a, Den
             int added = 0, any_more = 0;
             for (int w2 = 0; w2 < kDWaves; w2++) { added += (int)scan_tmp[8 + w2]; any_more |= (int)scan_tmp[16 + w2]; }
             if (added > 0) {
-                bitonic_sort_u64(sortbuf, y.sort_cap);
+                bitonic_sort_u64_by256(sortbuf, y.sort_cap);
                 topn = min(a.kcap, topn + added);
             } else {
                 __syncthreads();
@@ -518,6 +518,7 @@ __global__ __launch_bounds__(kDT, 2) void traverse_dense_kernel(QueryArgs a, Den
         auto run_tiles = [&](auto gtag) {
             typedef float v4f __attribute__((ext_vector_type(4)));
             constexpr int GL = decltype(gtag)::value;
+            constexpr int kInFlight = 16;                   // row reads under way per lane
             const int grp = lane / GL, sl = lane & (GL - 1);
             const int j = sl * 4;
             const bool has = j < a.dim;
@@ -554,17 +555,17 @@ __global__ __launch_bounds__(kDT, 2) void traverse_dense_kernel(QueryArgs a, Den
                     const uint16_t* cur = wl + list_pos;
                     float acc[GL];
 #pragma unroll
-                    for (int r0 = 0; r0 < GL; r0 += 8) {
-                        v4f x[8];
+                    for (int r0 = 0; r0 < GL; r0 += kInFlight) {
+                        v4f x[kInFlight];
 #pragma unroll
-                        for (int r = 0; r < 8; r++) {
+                        for (int r = 0; r < kInFlight; r++) {
                             // (lanes beyond the row's end read its head and add nothing: a load
                             //  under a condition would wait for the loads before it)
                             const int pt = (int)cur[min(grp * GL + r0 + r, nb - 1)];
                             x[r] = *reinterpret_cast<const v4f*>(base + pt * a.dim);
                         }
 #pragma unroll
-                        for (int r = 0; r < 8; r++) {
+                        for (int r = 0; r < kInFlight; r++) {
                             float s2 = 0.f;
                             float dd = x[r].x - q0; s2 = __builtin_fmaf(dd, dd, s2);
                             dd = x[r].y - q1; s2 = __builtin_fmaf(dd, dd, s2);
