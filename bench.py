@@ -87,6 +87,9 @@ def parse():
     p.add_argument("--build-reps", type=int, default=3)
     p.add_argument("--traversal", default="auto", choices=["auto", "step", "batch", "dense"])
     p.add_argument("--c5-batches", type=int, default=20, help="batches of the incremental workload")
+    p.add_argument("--append", default="auto", choices=["auto", "sort", "merge"],
+                   help="c5: how an append forms the new index (merge old slices with the sorted new "
+                        "points, or sort everything again)")
     p.add_argument("--copy-calibration", action="store_true",
                    help="also run a plain 1 GiB device copy (known HBM traffic) so that "
                         "rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE readings can be scaled")
@@ -159,6 +162,9 @@ def main():
     # ---- data and build ---------------------------------------------------------
     per_size = None
     if config == "c5":
+        _capi.check(lib.dcih_set_option(dci._dci_inst, _capi.OPT_APPEND,
+                                        {"auto": _capi.APPEND_AUTO, "sort": _capi.APPEND_SORT,
+                                         "merge": _capi.APPEND_MERGE}[a.append]))
         n_batch = a.n or shape["n"]
         Q = workloads.c5_queries(shape["nq"])
         if a.nq:
@@ -348,8 +354,9 @@ def main():
                  project_frac=build_bytes_proj / (proj_t * 1e-3) / 1e9 / HBM_PEAK_GBS,
                  segsort_frac=build_bytes_sort / (sort_t * 1e-3) / 1e9 / HBM_PEAK_GBS)
     if per_size is not None:
-        build["note"] = ("last append: %d new rows projected, all %d rows sorted; "
-                         "points_per_s counts the new rows" % (new_rows, N))
+        build["note"] = ("last append (mode %s): %d new rows projected, the index over all %d rows formed; "
+                         "points_per_s counts the new rows" % (a.append, new_rows, N))
+        build["append_mode"] = a.append
         build["total_points_per_s"] = N / build_wall
 
     # ---- extras: sweep of num_outer_iterations, blind querying ------------------------

@@ -14,6 +14,8 @@ CTR_VISITED, CTR_CANDIDATES, CTR_PROBES, CTR_STEPS = range(4)
 OPT_TRAVERSAL = 0
 OPT_DENSE_MIN_PROMOTIONS = 1
 OPT_FORGET_HINTS = 2
+OPT_APPEND = 3
+APPEND_AUTO, APPEND_SORT, APPEND_MERGE = 0, 1, 2
 TRAVERSAL_AUTO, TRAVERSAL_STEP, TRAVERSAL_BATCH, TRAVERSAL_DENSE = 0, 1, 2, 3
 NOALLOC_SCRATCH_BYTES = 32 << 20
 NUM_TIMERS = 7

@@ -132,6 +132,7 @@ struct dcih_index {
     int hint_k = 0, hint_outer = 0, hint_T = 0, hint_maxc = 0;   // query shape the hints belong to
     int traversal = 0;                  // DCIH_OPT_TRAVERSAL value
     int dense_min_promos = 384;         // DCIH_OPT_DENSE_MIN_PROMOTIONS value
+    int append_mode = 0;                // DCIH_OPT_APPEND value
     unsigned long long* d_phase_ticks = nullptr;   // optional profile of the batch kernel
     // grow-only workspace: query scratch, and the unsorted keys during a build
     void* ws = nullptr;
@@ -324,9 +325,11 @@ int dcih_set_directions(dcih_index* h, const float* h_dirs) {
 // arena `which`, which must already be large enough, and makes the result the handle's
 // index over the rows at d_data.  Synchronises the stream before returning; on failure the
 // handle's fields are untouched.
+// With merge_from > 0 the live index (over the first merge_from points, in the other arena) is
+// merged with the sorted new points instead of everything being sorted again.
 static int sort_into(dcih_index* h, int which, const float* d_keys, int64_t key_stride,
                      int64_t num_points, const float* d_data, int block_size, void* d_tmp,
-                     hipStream_t s) {
+                     hipStream_t s, int64_t merge_from = 0) {
     const int I = num_indices(h);
     const ArenaLayout y = arena_layout(I, num_points, block_size);
     char* base = (char*)h->arena[which];
@@ -339,7 +342,11 @@ static int sort_into(dcih_index* h, int which, const float* d_keys, int64_t key_
     int rc = zero_words64(hint, (int64_t)(((size_t)3 * block_size * sizeof(float) + 7) / 8), s);
     if (rc == DCIH_OK) {
         mark(h, DCIH_T_SEGSORT, 0, s);
-        rc = segsort(d_keys, key_stride, I, num_points, block_size, skeys, sids, inv, lids, d_tmp, s);
+        if (merge_from > 0)
+            rc = segsort_append(h->d_skeys, h->d_sids, merge_from, d_keys, key_stride, I, num_points, block_size,
+                                skeys, sids, inv, lids, d_tmp, s);
+        else
+            rc = segsort(d_keys, key_stride, I, num_points, block_size, skeys, sids, inv, lids, d_tmp, s);
         mark(h, DCIH_T_SEGSORT, 1, s);
     }
     // like the reference's dci_add, the call returns when the index is complete
@@ -426,7 +433,15 @@ int dcih_append(dcih_index* h, int dim, int64_t num_points, const float* d_data,
         ukeys = fresh_keys;
     }
     const int spare = 1 - h->cur;
-    const size_t tmp_bytes = segsort_tmp_bytes(I, total, block_size);
+    // Merging the old slices with the sorted new points instead of sorting everything again.
+    // Both are built; left to choose, the append sorts: the one-pass LDS sort moves 16 bytes per
+    // index entry, split + merge + inverse move 40, and on an MI355X the sort is the faster of the
+    // two at every size of the incremental workload (8.7 against 9.0 ms for 1M onto 19M points).
+    const bool merge = h->n > 0 && h->append_mode == 2 && h->d_inv != nullptr &&
+                       segsort_append_supported(h->n, total, block_size);
+    if (h->append_mode == 2 && h->n > 0 && !merge)
+        return fail(DCIH_EUNSUPPORTED, "dcih_append: this shape cannot be appended by merging (partitions too long)");
+    const size_t tmp_bytes = merge ? segsort_append_tmp_bytes(I, total) : segsort_tmp_bytes(I, total, block_size);
     int rc = ensure_arena(h, h->n > 0 ? spare : h->cur,
                           std::max(arena_layout(I, total, block_size).total,
                                    arena_layout(I, cap, block_size).total));
@@ -452,7 +467,7 @@ int dcih_append(dcih_index* h, int dim, int64_t num_points, const float* d_data,
     if (rc == DCIH_OK)
         // the partition boundaries move with the total, so every slice is formed again
         rc = sort_into(h, h->n > 0 ? spare : h->cur, ukeys, cap, total, rows, block_size,
-                       tmp_bytes ? h->ws : nullptr, s);
+                       tmp_bytes ? h->ws : nullptr, s, merge ? h->n : 0);
     else
         (void)hipStreamSynchronize(s);
     if (rc) {       // the index stays as it was
@@ -678,6 +693,10 @@ int dcih_set_option(dcih_index* h, int option, int value) {
     }
     if (option == DCIH_OPT_DENSE_MIN_PROMOTIONS && value >= 0) {
         h->dense_min_promos = value;
+        return DCIH_OK;
+    }
+    if (option == DCIH_OPT_APPEND && value >= 0 && value <= 2) {
+        h->append_mode = value;
         return DCIH_OK;
     }
     if (option == DCIH_OPT_FORGET_HINTS) {

@@ -24,6 +24,18 @@ int segsort(const float* d_keys, int64_t key_stride, int num_indices, int64_t n,
             float* d_skeys, int32_t* d_sids, uint16_t* d_inv, uint16_t* d_lids, void* d_tmp,
             hipStream_t s);
 
+// Appending: the index over n1 points from the sorted arrays of the index over their first
+// n0 points (same block_size) and the unsorted keys of the others (index i's key of point id
+// at d_keys + i * key_stride + id): old slices are split into runs of the new ones, the new
+// points sorted, the runs merged; nothing of the old part is sorted again.  Outputs as
+// segsort's; d_tmp = segsort_append_tmp_bytes() bytes.
+bool segsort_append_supported(int64_t n0, int64_t n1, int block_size);
+size_t segsort_append_tmp_bytes(int num_indices, int64_t n1);
+int segsort_append(const float* d_old_skeys, const int32_t* d_old_sids, int64_t n0,
+                   const float* d_keys, int64_t key_stride, int num_indices, int64_t n1, int block_size,
+                   float* d_skeys, int32_t* d_sids, uint16_t* d_inv, uint16_t* d_lids, void* d_tmp,
+                   hipStream_t s);
+
 struct QueryArgs {
     const float* skeys;      // [I][N] sorted projections
     const int32_t* sids;     // [I][N] point ids in the same order

@@ -11,6 +11,8 @@
 // write of the sorted keys and ids.  Longer slices are sorted tile by tile and
 // the tiles are then merged pairwise (merge path, staged through LDS), each
 // pass doubling the run length, the last one writing the final arrays.
+#include <algorithm>
+
 #include "common.h"
 #include "kernels.h"
 #include "radix_core.h"
@@ -29,6 +31,10 @@ struct SegGeom {
     int B;            // partitions
     int tiles;        // tiles per partition (by the longest partition)
     int tile_size;    // points per tile
+    // appending (radix kernel, packed output): only the points with ids from tail_from on are
+    // sorted, one run per partition from partition b_first on; -1 = everything
+    int64_t tail_from;
+    int b_first;
 };
 
 __device__ inline unsigned long long pack_key(float key, uint32_t pos) {
@@ -131,14 +137,16 @@ __global__ __launch_bounds__(kRadixThreads, (kRadixThreads == 256 && IPT > 45) ?
     // packed == null: the workgroup sorts a whole slice and writes the final arrays;
     // else it sorts one tile of a slice into packed (key, position in slice) words
     // for the merge passes
-    const int tiles = packed ? g.tiles : 1;
+    const bool tail = g.tail_from >= 0;
+    const int tiles = packed && !tail ? g.tiles : 1;
+    const int parts = tail ? g.B - g.b_first : g.B;
     const int tile = (int)(blockIdx.x % tiles);
-    const int b = (int)((blockIdx.x / tiles) % g.B);
-    const int64_t i = blockIdx.x / ((int64_t)tiles * g.B);
+    const int b = (int)((blockIdx.x / tiles) % parts) + (tail ? g.b_first : 0);
+    const int64_t i = blockIdx.x / ((int64_t)tiles * parts);
     const int64_t off = (int64_t)b * g.ppb;
-    const int64_t t0 = packed ? (int64_t)tile * g.tile_size : 0;
+    const int64_t t0 = tail ? max((int64_t)0, g.tail_from - off) : (packed ? (int64_t)tile * g.tile_size : 0);
     const int64_t nseg = min(g.n - off, g.ppb) - t0;
-    const int n = (int)(packed ? min(nseg, (int64_t)g.tile_size) : nseg);
+    const int n = (int)(packed && !tail ? min(nseg, (int64_t)g.tile_size) : nseg);
     if (n <= 0) return;
     const int64_t base = i * g.n + off + t0;
     const int64_t kbase = i * g.kstride + off + t0;
@@ -235,7 +243,8 @@ static int launch_radix(const float* d_keys, const SegGeom& g, int num_indices, 
         });
         if (rc) return rc;
     }
-    const int64_t blocks = (int64_t)num_indices * g.B * (d_packed ? g.tiles : 1);
+    const int64_t blocks = g.tail_from >= 0 ? (int64_t)num_indices * (g.B - g.b_first)
+                                            : (int64_t)num_indices * g.B * (d_packed ? g.tiles : 1);
     if (blocks > 0x7fffffffLL) return fail(-1, "segsort: too many slices for one launch");
     hipLaunchKernelGGL((segsort_radix_kernel<NT, IPT>), dim3((unsigned)blocks), dim3(NT), lds, s,
                        d_keys, g, d_skeys, d_sids, d_inv, d_lids, d_packed);
@@ -264,21 +273,81 @@ __device__ inline int64_t merge_split_wave(const unsigned long long* __restrict_
     return lo;
 }
 
+// Outputs [d0, d1) (at most kMergeChunk of them) of the merge of the sorted runs A (la words)
+// and Bv (lb words), A winning ties, by one workgroup: two wavefronts find where the piece
+// starts and ends in either run, the two pieces are read into LDS with coalesced loads, every
+// thread merges kMergeItems outputs there, and the outputs leave in coalesced stores, either
+// as packed words to dst + out0 or, for the last pass (skeys != null), as the final arrays of
+// the slice that starts at element `base` of its index and at point id `off`; out0 is then
+// the first output's position inside the slice.
+struct MergeScratch {
+    unsigned long long in[kMergeChunk];
+    unsigned long long out[kMergeChunk];
+    int64_t split[2];
+};
+__device__ inline void merge_piece(MergeScratch& ms, const unsigned long long* __restrict__ A, int64_t la,
+                                   const unsigned long long* __restrict__ Bv, int64_t lb, int64_t d0, int64_t d1,
+                                   unsigned long long* __restrict__ dst, int64_t out0, int64_t base, int64_t off,
+                                   float* __restrict__ skeys, int32_t* __restrict__ sids,
+                                   uint16_t* __restrict__ inv, uint16_t* __restrict__ lids) {
+    const int tid = threadIdx.x, lane = tid & (kWave - 1), wave = tid / kWave;
+    const int cnt = (int)(d1 - d0);
+    if (wave < 2) {
+        const int64_t sp = merge_split_wave(A, la, Bv, lb, wave ? d1 : d0, lane);
+        if (lane == 0) ms.split[wave] = sp;
+    }
+    __syncthreads();
+    const int64_t ia0 = ms.split[0], ia1 = ms.split[1];
+    const int64_t ib0 = d0 - ia0;
+    const int na = (int)(ia1 - ia0), nb = cnt - na;
+    for (int j = tid; j < cnt; j += kMergeThreads)
+        ms.in[j] = j < na ? A[ia0 + j] : Bv[ib0 + (j - na)];
+    __syncthreads();
+    {
+        const unsigned long long* LA = ms.in;
+        const unsigned long long* LB = ms.in + na;
+        const int d = tid * kMergeItems;
+        if (d < cnt) {
+            int lo = max(0, d - nb), hi = min(d, na);
+            while (lo < hi) {
+                const int a = (lo + hi) >> 1;
+                if (LA[a] < LB[d - 1 - a]) lo = a + 1; else hi = a;
+            }
+            int ia = lo, ib = d - lo;
+            const int m = min(kMergeItems, cnt - d);
+            unsigned long long va = ia < na ? LA[ia] : ~0ull;
+            unsigned long long vb = ib < nb ? LB[ib] : ~0ull;
+            for (int t = 0; t < m; t++) {
+                const bool takeA = ib >= nb || (ia < na && va < vb);
+                if (takeA) { ms.out[d + t] = va; ia++; va = ia < na ? LA[ia] : ~0ull; }
+                else       { ms.out[d + t] = vb; ib++; vb = ib < nb ? LB[ib] : ~0ull; }
+            }
+        }
+    }
+    __syncthreads();
+    if (!skeys) {
+        for (int j = tid; j < cnt; j += kMergeThreads) dst[base + out0 + j] = ms.out[j];
+    } else {
+        for (int j = tid; j < cnt; j += kMergeThreads) {
+            const unsigned long long w = ms.out[j];
+            const int64_t e = base + out0 + j;
+            skeys[e] = ord2f((uint32_t)(w >> 32));
+            sids[e] = (int32_t)(off + (uint32_t)w);
+            if (inv) inv[base + (uint32_t)w] = (uint16_t)(out0 + j);
+            if (lids) lids[e] = (uint16_t)(uint32_t)w;
+        }
+    }
+}
+
 // One merge pass: within every slice, neighbouring sorted runs of length `run`
-// (a multiple of kMergeChunk / 2) are merged into runs of 2*run.  A workgroup
-// produces kMergeChunk outputs: two wavefronts find where its piece starts and
-// ends in either run, the two pieces are read into LDS with coalesced loads,
-// every thread merges kMergeItems outputs there, and the outputs leave in
-// coalesced stores.  The last pass (skeys != null) writes the final arrays
-// instead of packed words.
+// (a multiple of kMergeChunk / 2) are merged into runs of 2*run; a workgroup
+// produces kMergeChunk outputs.  The last pass (skeys != null) writes the final
+// arrays instead of packed words.
 __global__ __launch_bounds__(kMergeThreads) void segsort_merge_kernel(
     const unsigned long long* __restrict__ src, unsigned long long* __restrict__ dst,
     SegGeom g, int chunks, int64_t run, float* __restrict__ skeys, int32_t* __restrict__ sids,
     uint16_t* __restrict__ inv, uint16_t* __restrict__ lids) {
-    __shared__ unsigned long long s_in[kMergeChunk];
-    __shared__ unsigned long long s_out[kMergeChunk];
-    __shared__ int64_t s_split[2];
-    const int tid = threadIdx.x, lane = tid & (kWave - 1), wave = tid / kWave;
+    __shared__ MergeScratch ms;
     const int64_t flat = blockIdx.x;
     const int chunk = (int)(flat % chunks);
     const int b = (int)((flat / chunks) % g.B);
@@ -293,56 +362,129 @@ __global__ __launch_bounds__(kMergeThreads) void segsort_merge_kernel(
     const int64_t a0 = ps, a1 = min(ps + run, nseg);
     const int64_t b0 = a1, b1 = min(ps + 2 * run, nseg);
     const int64_t la = a1 - a0, lb = b1 - b0;
-    const unsigned long long* A = src + base + a0;
-    const unsigned long long* Bv = src + base + b0;
     const int64_t d0 = o0 - ps;                               // first output of this workgroup
     const int64_t d1 = min(d0 + kMergeChunk, la + lb);
-    const int cnt = (int)(d1 - d0);
-    if (wave < 2) {
-        const int64_t sp = merge_split_wave(A, la, Bv, lb, wave ? d1 : d0, lane);
-        if (lane == 0) s_split[wave] = sp;
-    }
-    __syncthreads();
-    const int64_t ia0 = s_split[0], ia1 = s_split[1];
-    const int64_t ib0 = d0 - ia0;
-    const int na = (int)(ia1 - ia0), nb = cnt - na;
-    for (int j = tid; j < cnt; j += kMergeThreads)
-        s_in[j] = j < na ? A[ia0 + j] : Bv[ib0 + (j - na)];
-    __syncthreads();
-    {
-        const unsigned long long* LA = s_in;
-        const unsigned long long* LB = s_in + na;
-        const int d = tid * kMergeItems;
-        if (d < cnt) {
-            int lo = max(0, d - nb), hi = min(d, na);
-            while (lo < hi) {
-                const int a = (lo + hi) >> 1;
-                if (LA[a] < LB[d - 1 - a]) lo = a + 1; else hi = a;
-            }
-            int ia = lo, ib = d - lo;
-            const int m = min(kMergeItems, cnt - d);
-            unsigned long long va = ia < na ? LA[ia] : ~0ull;
-            unsigned long long vb = ib < nb ? LB[ib] : ~0ull;
-            for (int t = 0; t < m; t++) {
-                const bool takeA = ib >= nb || (ia < na && va < vb);
-                if (takeA) { s_out[d + t] = va; ia++; va = ia < na ? LA[ia] : ~0ull; }
-                else       { s_out[d + t] = vb; ib++; vb = ib < nb ? LB[ib] : ~0ull; }
-            }
+    merge_piece(ms, src + base + a0, la, src + base + b0, lb, d0, d1, dst, ps + d0, base, off,
+                skeys, sids, inv, lids);
+}
+
+// ---------------------------------------------------------------------------
+// Appending points to a built index without sorting the old ones again.
+// The partitions are the id ranges [b * ppb, (b + 1) * ppb) with ppb = ceil(n / B), so
+// n0 -> n1 points moves every boundary (p0 -> p1 points per partition), and a new slice is
+// made of pieces of old slices plus, in the last partitions, new points:
+//   * an old slice is shorter than a new one, so it contributes to at most two new slices,
+//     to each a contiguous range of its ids; taking those ids out of the slice in their
+//     sorted order (a stable split in two) gives two sorted runs;
+//   * the new points of a partition are sorted on their own (LDS radix sort): one more run;
+//   * the runs of a new slice, laid end to end by ascending ids, are merged pairwise
+//     (merge path, as in the build of long slices), the last pass writing the final arrays.
+// Run r of new slice b starts at position run_start(b, r) of the slice; all of it follows
+// from n0, n1, p0, p1 alone.
+struct AppendGeom {
+    int64_t n0, n1;     // points before and after
+    int64_t p0, p1;     // points per partition before and after
+    int B;
+};
+__host__ __device__ inline int64_t slice_len(const AppendGeom& g, int b) {
+    const int64_t v = g.n1 - (int64_t)b * g.p1;
+    return v < 0 ? 0 : (v < g.p1 ? v : g.p1);
+}
+__host__ __device__ inline int64_t old_in_slice(const AppendGeom& g, int b) {     // its points with ids below n0
+    const int64_t v = g.n0 - (int64_t)b * g.p1, len = slice_len(g, b);
+    return v < 0 ? 0 : (v < len ? v : len);
+}
+__host__ __device__ inline int slice_runs(const AppendGeom& g, int b) {
+    const int64_t lo = (int64_t)b * g.p1, n_old = old_in_slice(g, b), len = slice_len(g, b);
+    const int r_old = n_old > 0 ? (int)((lo + n_old - 1) / g.p0 - lo / g.p0 + 1) : 0;
+    return r_old + (len > n_old ? 1 : 0);
+}
+__host__ __device__ inline int64_t run_start(const AppendGeom& g, int b, int r) {
+    const int64_t lo = (int64_t)b * g.p1, n_old = old_in_slice(g, b), len = slice_len(g, b);
+    const int r_old = n_old > 0 ? (int)((lo + n_old - 1) / g.p0 - lo / g.p0 + 1) : 0;
+    if (r <= 0) return 0;
+    if (r < r_old) return (lo / g.p0 + r) * g.p0 - lo;
+    if (r == r_old) return n_old;
+    return len;
+}
+
+// Stable split of every old slice: its (key, id) pairs leave, in their sorted order, for the
+// runs of the one or two new slices their ids fall into, as packed (key, position in the new
+// slice) words.  One workgroup per (simple index, old slice).
+constexpr int kSplitThreads = 256;
+__global__ __launch_bounds__(kSplitThreads) void append_split_kernel(
+    const float* __restrict__ old_keys, const int32_t* __restrict__ old_ids, AppendGeom g,
+    unsigned long long* __restrict__ packed) {
+    __shared__ int s_wave[kSplitThreads / kWave][2];
+    const int old_slices = (int)((g.n0 + g.p0 - 1) / g.p0);
+    const int a = (int)(blockIdx.x % old_slices);
+    const int64_t i = blockIdx.x / old_slices;
+    const int64_t lo = (int64_t)a * g.p0;
+    const int len = (int)min(g.p0, g.n0 - lo);
+    const int d0 = (int)(lo / g.p1);
+    const int64_t cut = (int64_t)(d0 + 1) * g.p1;                // ids from here on go to slice d0 + 1
+    // where the two runs start: ids ascend along a new slice's runs
+    const int64_t out_lo = i * g.n1 + (int64_t)d0 * g.p1 + (lo - (int64_t)d0 * g.p1);
+    const int64_t out_hi = i * g.n1 + cut;                       // the next slice's first run
+    const float* keys = old_keys + i * g.n0 + lo;
+    const int32_t* ids = old_ids + i * g.n0 + lo;
+    const int tid = threadIdx.x, lane = tid & (kWave - 1), wave = tid / kWave;
+    int done_lo = 0, done_hi = 0;
+    for (int j0 = 0; j0 < len; j0 += kSplitThreads) {
+        const int j = j0 + tid;
+        const bool real = j < len;
+        const int64_t id = real ? (int64_t)ids[j] : 0;
+        const uint32_t ok = real ? f2ord(keys[j]) : 0u;
+        const bool hi = real && id >= cut;
+        const unsigned long long m_hi = __ballot(hi), m_lo = __ballot(real && !hi);
+        const unsigned long long below = (1ull << lane) - 1ull;
+        if (lane == 0) { s_wave[wave][0] = __popcll(m_lo); s_wave[wave][1] = __popcll(m_hi); }
+        __syncthreads();
+        int before_lo = done_lo, before_hi = done_hi, all_lo = 0, all_hi = 0;
+        for (int w = 0; w < kSplitThreads / kWave; w++) {
+            if (w < wave) { before_lo += s_wave[w][0]; before_hi += s_wave[w][1]; }
+            all_lo += s_wave[w][0]; all_hi += s_wave[w][1];
         }
-    }
-    __syncthreads();
-    const int64_t out0 = base + ps + d0;
-    if (!skeys) {
-        for (int j = tid; j < cnt; j += kMergeThreads) dst[out0 + j] = s_out[j];
-    } else {
-        for (int j = tid; j < cnt; j += kMergeThreads) {
-            const unsigned long long w = s_out[j];
-            const int64_t e = out0 + j;
-            skeys[e] = ord2f((uint32_t)(w >> 32));
-            sids[e] = (int32_t)(off + (uint32_t)w);
-            if (inv) inv[base + (uint32_t)w] = (uint16_t)(ps + d0 + j);
-            if (lids) lids[e] = (uint16_t)(uint32_t)w;
+        if (real) {
+            if (hi) packed[out_hi + before_hi + __popcll(m_hi & below)] = ((unsigned long long)ok << 32) | (uint32_t)(id - cut);
+            else packed[out_lo + before_lo + __popcll(m_lo & below)] = ((unsigned long long)ok << 32) | (uint32_t)(id - (int64_t)d0 * g.p1);
         }
+        done_lo += all_lo; done_hi += all_hi;
+        __syncthreads();
+    }
+}
+
+// One pass over the runs of every new slice: runs 2q * step and (2q + 1) * step of level 0
+// (each already a union of `step` original runs) are merged.  A workgroup produces the
+// outputs [chunk * kMergeChunk, ...) of its slice, pair by pair where they straddle pairs.
+// A slice whose runs this pass brings down to one gets its final arrays written at once, and
+// later passes skip it: most slices have two runs and are done after the first pass.
+__global__ __launch_bounds__(kMergeThreads) void append_merge_kernel(
+    const unsigned long long* __restrict__ src, unsigned long long* __restrict__ dst, AppendGeom g,
+    int chunks, int step, float* __restrict__ skeys, int32_t* __restrict__ sids,
+    uint16_t* __restrict__ inv, uint16_t* __restrict__ lids) {
+    __shared__ MergeScratch ms;
+    const int64_t flat = blockIdx.x;
+    const int chunk = (int)(flat % chunks);
+    const int b = (int)((flat / chunks) % g.B);
+    const int64_t i = flat / ((int64_t)chunks * g.B);
+    const int64_t off = (int64_t)b * g.p1;
+    const int64_t nseg = slice_len(g, b);
+    const int64_t o0 = (int64_t)chunk * kMergeChunk, o1 = min(o0 + kMergeChunk, nseg);
+    if (o0 >= nseg) return;
+    const int64_t base = i * g.n1 + off;
+    const int runs = slice_runs(g, b);
+    if (step > 1 && step >= runs) return;                    // an earlier pass finished this slice
+    if (2 * step < runs) skeys = nullptr;                    // more passes to come: packed words
+    for (int q = 0; 2 * q * step < runs; q++) {
+        const int64_t a0 = run_start(g, b, 2 * q * step), a1 = run_start(g, b, (2 * q + 1) * step);
+        const int64_t b1 = run_start(g, b, (2 * q + 2) * step);
+        if (b1 <= o0) continue;
+        if (a0 >= o1) break;
+        const int64_t d0 = max(o0, a0) - a0, d1 = min(o1, b1) - a0;       // this pair's outputs of this workgroup
+        merge_piece(ms, src + base + a0, a1 - a0, src + base + a1, b1 - a1, d0, d1, dst, a0 + d0, base, off,
+                    skeys, sids, inv, lids);
+        __syncthreads();
     }
 }
 
@@ -370,6 +512,8 @@ int segsort(const float* d_keys, int64_t key_stride, int num_indices, int64_t n,
     g.ppb = (n + block_size - 1) / block_size;
     g.tiles = (int)((g.ppb + kTileCap - 1) / kTileCap);
     g.tile_size = kTileCap;
+    g.tail_from = -1;
+    g.b_first = 0;
     const int np2 = next_pow2((int)min((int64_t)kTileCap, g.ppb));
     // at most kTileCap / 1024 elements per thread (the inverse-permutation pass relies on it)
     const int threads = max(64, min(1024, np2 / 2));
@@ -435,6 +579,102 @@ int segsort(const float* d_keys, int64_t key_stride, int num_indices, int64_t n,
         unsigned long long* t = bufA; bufA = bufB; bufB = t;
     }
     DCIH_HIP(hipGetLastError());
+    return 0;
+}
+
+// inv[point] = position of the point inside its sorted slice, from the slice's local ids.
+__global__ __launch_bounds__(512) void slice_inverse_kernel(const uint16_t* __restrict__ lids,
+                                                            uint16_t* __restrict__ inv, int64_t n, int64_t ppb, int B) {
+    extern __shared__ uint16_t pos_of[];
+    const int b = (int)(blockIdx.x % B);
+    const int64_t i = blockIdx.x / B;
+    const int64_t off = (int64_t)b * ppb;
+    const int len = (int)min(ppb, n - off);
+    if (len <= 0) return;
+    const int64_t base = i * n + off;
+    for (int j = threadIdx.x; j < len; j += blockDim.x) pos_of[lids[base + j]] = (uint16_t)j;
+    __syncthreads();
+    for (int j = threadIdx.x; j < len; j += blockDim.x) inv[base + j] = pos_of[j];
+}
+
+// ---- appending -------------------------------------------------------------------
+bool segsort_append_supported(int64_t n0, int64_t n1, int block_size) {
+    if (n0 <= 0 || n1 <= n0 || block_size < 1) return false;
+    const int64_t p0 = (n0 + block_size - 1) / block_size, p1 = (n1 + block_size - 1) / block_size;
+    // the new points of a partition are sorted by one LDS pass; positions fit 16 bits
+    return p1 <= kRadixMax && p1 <= 65536 && p0 <= p1;
+}
+
+size_t segsort_append_tmp_bytes(int num_indices, int64_t n1) {
+    return (size_t)2 * num_indices * n1 * sizeof(unsigned long long);
+}
+
+int segsort_append(const float* d_old_skeys, const int32_t* d_old_sids, int64_t n0,
+                   const float* d_keys, int64_t key_stride, int num_indices, int64_t n1, int block_size,
+                   float* d_skeys, int32_t* d_sids, uint16_t* d_inv, uint16_t* d_lids, void* d_tmp,
+                   hipStream_t s) {
+    if (!segsort_append_supported(n0, n1, block_size)) return fail(-1, "segsort_append: shape not supported");
+    if (!d_tmp) return fail(-1, "segsort_append: scratch buffer missing");
+    AppendGeom ag;
+    ag.n0 = n0; ag.n1 = n1; ag.B = block_size;
+    ag.p0 = (n0 + block_size - 1) / block_size;
+    ag.p1 = (n1 + block_size - 1) / block_size;
+    unsigned long long* bufA = (unsigned long long*)d_tmp;
+    unsigned long long* bufB = bufA + (size_t)num_indices * n1;
+    // 1. the old slices' entries, split into the runs of the new slices
+    const int64_t old_slices = (n0 + ag.p0 - 1) / ag.p0;
+    if (num_indices * old_slices > 0x7fffffffLL) return fail(-1, "segsort_append: too many slices for one launch");
+    hipLaunchKernelGGL(append_split_kernel, dim3((unsigned)(num_indices * old_slices)), dim3(kSplitThreads), 0, s,
+                       d_old_skeys, d_old_sids, ag, bufA);
+    DCIH_HIP(hipGetLastError());
+    // 2. the new points of every partition that has some, sorted into one more run
+    {
+        SegGeom g;
+        g.kstride = key_stride; g.n = n1; g.B = block_size; g.ppb = ag.p1;
+        g.tiles = 1; g.tile_size = 0;
+        g.tail_from = n0;
+        g.b_first = (int)(n0 / ag.p1);
+        int64_t longest = 0;                               // longest run of new points in one partition
+        for (int b = g.b_first; b < block_size; b++)
+            longest = std::max(longest, slice_len(ag, b) - old_in_slice(ag, b));
+        int rc = -1;
+#define DCIH_RADIX_TAIL(NT, IPT) \
+    if (rc < 0 && longest <= (int64_t)(NT) * (IPT))  \
+        rc = launch_radix<NT, IPT>(d_keys, g, num_indices, nullptr, nullptr, nullptr, nullptr, bufA, s)
+        DCIH_RADIX_TAIL(64, 9); DCIH_RADIX_TAIL(64, 33); DCIH_RADIX_TAIL(128, 33); DCIH_RADIX_TAIL(256, 33);
+        DCIH_RADIX_TAIL(256, 57); DCIH_RADIX_TAIL(512, 39); DCIH_RADIX_TAIL(512, 51); DCIH_RADIX_TAIL(512, 63);
+#undef DCIH_RADIX_TAIL
+        if (rc) return rc < 0 ? fail(-1, "segsort_append: no radix configuration for the new points") : rc;
+    }
+    // 3. pairwise merges of every slice's runs
+    int most_runs = 1;
+    for (int b = 0; b < block_size; b++) most_runs = std::max(most_runs, slice_runs(ag, b));
+    const int chunks = (int)((ag.p1 + kMergeChunk - 1) / kMergeChunk);
+    const int64_t mblocks = (int64_t)num_indices * block_size * chunks;
+    if (mblocks > 0x7fffffffLL) return fail(-1, "segsort_append: too many merge chunks for one launch");
+    for (int step = 1;; step *= 2) {
+        const bool last = 2 * step >= most_runs;
+        hipLaunchKernelGGL(append_merge_kernel, dim3((unsigned)mblocks), dim3(kMergeThreads), 0, s,
+                           bufA, bufB, ag, chunks, step, d_skeys, d_sids, (uint16_t*)nullptr, d_lids);
+        unsigned long long* t = bufA; bufA = bufB; bufB = t;
+        if (last) break;
+    }
+    DCIH_HIP(hipGetLastError());
+    // 4. the inverse permutation of every slice from its local ids, turned round in LDS so that
+    // reads and writes are coalesced (written from the merge it would be a scatter of 2-byte words)
+    if (d_inv) {
+        const size_t lds = (size_t)ag.p1 * sizeof(uint16_t);
+        static DeviceOnce once;
+        const int rc = once.run([]() -> int {
+            DCIH_HIP(hipFuncSetAttribute((const void*)slice_inverse_kernel,
+                                         hipFuncAttributeMaxDynamicSharedMemorySize, 65536 * (int)sizeof(uint16_t)));
+            return 0;
+        });
+        if (rc) return rc;
+        hipLaunchKernelGGL(slice_inverse_kernel, dim3((unsigned)((int64_t)num_indices * block_size)), dim3(512), lds, s,
+                           d_lids, d_inv, n1, ag.p1, block_size);
+        DCIH_HIP(hipGetLastError());
+    }
     return 0;
 }
 

@@ -69,8 +69,13 @@ enum {
  * DCIH_OPT_FORGET_HINTS (value ignored): drops what earlier queries taught the
  * handle about where traversals stop (used only to size the batch kernel's
  * epochs, never visible in results), so that the next call runs like a first one.
+ * DCIH_OPT_APPEND: how dcih_append forms the new index: 0 = automatic (today: sorts,
+ * the faster of the two wherever it was measured), 1 = sort all projections again
+ * (only the new rows are projected), 2 = merge: the old slices are split into sorted
+ * runs of the new ones, the new points sorted, the runs merged (error where the shape
+ * does not allow it: partitions of more than 32256 points).  All give the same index.
  */
-enum { DCIH_OPT_TRAVERSAL = 0, DCIH_OPT_DENSE_MIN_PROMOTIONS = 1, DCIH_OPT_FORGET_HINTS = 2 };
+enum { DCIH_OPT_TRAVERSAL = 0, DCIH_OPT_DENSE_MIN_PROMOTIONS = 1, DCIH_OPT_FORGET_HINTS = 2, DCIH_OPT_APPEND = 3 };
 
 /* Message for the last failing call on this thread ("" if none). */
 const char* dcih_last_error(void);
