@@ -378,6 +378,12 @@ int query(const QueryArgs& a_in, hipStream_t s, hipEvent_t* ev, bool* ran) {
         return fail(-4, "query: this shape does not fit the batch traversal kernel");
     if (a.mode == 3 && !can_dense)
         return fail(-4, "query: this shape does not fit the dense traversal kernel");
+    // Left to choose: the stop rule needs k promotions by a window's first lane, which takes
+    // about k * T promotions in all; from the number at which the dense kernel is the cheaper
+    // one, every item goes straight to it (no hints needed: also a first call is routed right).
+    if (a.mode == 0 && can_dense && !a.blind && a.dense_min_promos > 0 &&
+        (int64_t)a.k_stop * a.T >= (int64_t)a.dense_min_promos)
+        a.mode = 3;
     const bool use_block = a.mode != 1 && a.mode != 3 && can_block;
     // the batch kernel hands items that need many promotions to the dense kernel
     if (!(use_block && a.mode == 0 && can_dense && a.dense_items && a.dense_min_promos > 0)) {
