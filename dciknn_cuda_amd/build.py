@@ -78,8 +78,34 @@ def build_extension(verbose=False):
     return EXT
 
 
+STAMP = os.path.join(HERE, "build_stamp.txt")
+
+
+def source_digest():
+    """Hash of every source file the two libraries are built from."""
+    import hashlib
+    h = hashlib.sha256()
+    for name in sorted(os.listdir(CSRC)):
+        if name.endswith((".hip", ".h", ".cpp")):
+            with open(os.path.join(CSRC, name), "rb") as f:
+                h.update(name.encode() + b"\0" + f.read())
+    return h.hexdigest()
+
+
 def build_all(verbose=False):
-    return build_library(verbose), build_extension(verbose)
+    out = build_library(verbose), build_extension(verbose)
+    with open(STAMP, "w") as f:
+        f.write(source_digest() + "\n")
+    return out
+
+
+def is_stale():
+    """True when the libraries were built from other sources than the tree holds now."""
+    try:
+        with open(STAMP) as f:
+            return f.read().strip() != source_digest()
+    except OSError:
+        return False      # no stamp: built by other means, nothing to compare with
 
 
 def ensure_built():
@@ -87,6 +113,9 @@ def ensure_built():
     this; they never rebuild what is there)."""
     if not (os.path.exists(LIB) and os.path.exists(EXT)):
         build_all()
+    elif is_stale():
+        print("dciknn_cuda_amd: libdci_hip.so / _dci_cuda.so are older than the sources in csrc/; "
+              "run `python -m dciknn_cuda_amd.build` to test what the tree holds", file=sys.stderr)
     return LIB, EXT
 
 
