@@ -252,6 +252,193 @@ static int launch_radix(const float* d_keys, const SegGeom& g, int num_indices, 
     return 0;
 }
 
+
+// ---------------------------------------------------------------------------
+// The same sort moving ONE word per item: (16 key bits << 16 | id).  Four passes order the
+// items by the low half of their keys, then every item fetches the high half of its key by id
+// (the slice was read a moment ago and sits in L2) and four more passes order by that; LSD
+// passes are stable, so the result is ordered by (key, id).  Half the scatters and reads of the
+// two-word kernel, half the registers, and with the digit counters inside the staging buffer a
+// slice takes 4 bytes of LDS per point: two workgroups share a CU up to 20 k points, and one's
+// barrier-separated phases overlap the other's.  Destinations come from a second round of
+// returning atomics on the scanned counters (no separate rank table), held two to a register
+// until every thread has its own (the scatter overwrites the counters).
+template <int NT, int IPT>
+__device__ inline void lds_radix_half(uint32_t (&w)[IPT], uint32_t* stage, uint32_t* misc, uint32_t varying16) {
+    const int tid = threadIdx.x;
+    const int lane = tid & 63, wave = tid >> 6;
+    uint32_t* cnt32 = stage;                                   // [16][NT] 16-bit counters, digit-major
+    const uint32_t half = (uint32_t)(tid & 1) * 16u;
+    for (int shift = 16; shift < 32; shift += 4) {
+        if (((varying16 >> (shift - 16)) & 15u) == 0u) continue;     // same nibble everywhere
+        __syncthreads();
+#pragma unroll
+        for (int q = 0; q < 8; q++) cnt32[tid + q * NT] = 0;
+        __syncthreads();
+#pragma unroll
+        for (int r = 0; r < IPT; r++) {
+            const uint32_t a = ((w[r] >> shift) & 15u) * NT + tid;
+            atomicAdd(&cnt32[a >> 1], 1u << half);
+        }
+        __syncthreads();
+        {   // exclusive scan of the 16 * NT counters in memory order
+            uint32_t v[8];
+            uint32_t sum = 0;
+#pragma unroll
+            for (int q = 0; q < 8; q++) { v[q] = cnt32[tid * 8 + q]; sum += (v[q] & 0xffffu) + (v[q] >> 16); }
+            uint32_t incl = sum;
+#pragma unroll
+            for (int o = 1; o < 64; o <<= 1) {
+                const uint32_t t = (uint32_t)__shfl_up((int)incl, o, 64);
+                if (lane >= o) incl += t;
+            }
+            if (lane == 63) misc[wave] = incl;
+            __syncthreads();
+            uint32_t run = incl - sum;
+            for (int w2 = 0; w2 < wave; w2++) run += misc[w2];
+#pragma unroll
+            for (int q = 0; q < 8; q++) {
+                const uint32_t lo = v[q] & 0xffffu, hi = v[q] >> 16;
+                cnt32[tid * 8 + q] = run | ((run + lo) << 16);
+                run += lo + hi;
+            }
+        }
+        __syncthreads();
+        uint32_t dst[(IPT + 1) / 2];                           // destinations, two to a register
+        {
+            int shift2 = shift;
+            asm volatile("" : "+s"(shift2));
+#pragma unroll
+            for (int r = 0; r < IPT; r++) {
+                const uint32_t a = ((w[r] >> shift2) & 15u) * NT + tid;
+                const uint32_t d = (atomicAdd(&cnt32[a >> 1], 1u << half) >> half) & 0xffffu;
+                if (r & 1) dst[r >> 1] |= d << 16; else dst[r >> 1] = d;
+                if ((r & 7) == 7) __builtin_amdgcn_sched_barrier(0);
+            }
+        }
+        __syncthreads();
+#pragma unroll
+        for (int r = 0; r < IPT; r++) {
+            stage[(r & 1) ? (dst[r >> 1] >> 16) : (dst[r >> 1] & 0xffffu)] = w[r];
+            if ((r & 7) == 7) __builtin_amdgcn_sched_barrier(0);
+        }
+        __syncthreads();
+#pragma unroll
+        for (int r = 0; r < IPT; r++) {
+            w[r] = stage[tid * IPT + r];
+            if ((r & 7) == 7) __builtin_amdgcn_sched_barrier(0);
+        }
+    }
+}
+
+template <int NT, int IPT, int WPS>
+__global__ __launch_bounds__(NT, WPS) void segsort_radix1w_kernel(
+    const float* __restrict__ keys, SegGeom g, float* __restrict__ skeys,
+    int32_t* __restrict__ sids, uint16_t* __restrict__ inv, uint16_t* __restrict__ lids) {
+    extern __shared__ uint32_t rs[];
+    uint32_t* stage = rs;                                         // IPT * NT words (>= 8 * NT)
+    uint16_t* stage16 = reinterpret_cast<uint16_t*>(rs);
+    uint32_t* misc = rs + IPT * NT;                               // 64 words
+    const int tid = threadIdx.x;
+    const int lane = tid & 63;
+    const int b = (int)(blockIdx.x % g.B);
+    const int64_t i = blockIdx.x / g.B;
+    const int64_t off = (int64_t)b * g.ppb;
+    const int n = (int)min(g.n - off, g.ppb);
+    if (n <= 0) return;
+    const int64_t base = i * g.n + off;
+    const float* kin = keys + i * g.kstride + off;
+
+    if (tid < 2) misc[32 + tid] = tid ? 0xffffffffu : 0u;        // OR / AND of all keys
+    uint32_t w[IPT];
+    {   // coalesced reads, all in flight at once; (low key half, position) words through LDS into
+        // the blocked arrangement; pads sort last and stay last
+        uint32_t vor = 0, vand = 0xffffffffu;
+#pragma unroll
+        for (int r = 0; r < IPT; r++) w[r] = __builtin_bit_cast(uint32_t, kin[min(r * NT + tid, n - 1)]);
+#pragma unroll
+        for (int r = 0; r < IPT; r++) {
+            const int j = r * NT + tid;
+            const uint32_t o = f2ord(__builtin_bit_cast(float, w[r]) + 0.0f);
+            vor |= j < n ? o : 0u;
+            vand &= j < n ? o : 0xffffffffu;
+            stage[j] = j < n ? ((o << 16) | (uint32_t)j) : (0xffff0000u | (uint32_t)(j & 0xffff));
+        }
+        for (int o = 32; o > 0; o >>= 1) {
+            vor |= (uint32_t)__shfl_xor((int)vor, o, 64);
+            vand &= (uint32_t)__shfl_xor((int)vand, o, 64);
+        }
+        if (lane == 0) { atomicOr(&misc[32], vor); atomicAnd(&misc[33], vand); }
+    }
+    __syncthreads();
+    const uint32_t varying = misc[32] ^ misc[33];
+#pragma unroll
+    for (int r = 0; r < IPT; r++) w[r] = stage[tid * IPT + r];
+
+    lds_radix_half<NT, IPT>(w, stage, misc, varying & 0xffffu);
+    // the other half of every key, by id (the first n sorted items are the real ones); the
+    // slice was read a moment ago and sits in L2
+#pragma unroll
+    for (int r = 0; r < IPT; r++) {
+        const uint32_t id = w[r] & 0xffffu;
+        const bool real = tid * IPT + r < n;
+        const float kv = kin[real ? id : 0];
+        const uint32_t o = f2ord(kv + 0.0f);
+        w[r] = real ? ((o & 0xffff0000u) | id) : (0xffff0000u | id);
+    }
+    lds_radix_half<NT, IPT>(w, stage, misc, varying >> 16);
+
+    // results, through LDS so that every global write is coalesced: keys (fetched whole by id), ids
+    uint32_t full[IPT];
+#pragma unroll
+    for (int r = 0; r < IPT; r++) {
+        const bool real = tid * IPT + r < n;
+        full[r] = f2ord(kin[real ? (w[r] & 0xffffu) : 0] + 0.0f);
+    }
+    __syncthreads();
+#pragma unroll
+    for (int r = 0; r < IPT; r++) stage[tid * IPT + r] = full[r];
+    __syncthreads();
+    for (int j = tid; j < n; j += NT) skeys[base + j] = ord2f(stage[j]);
+    __syncthreads();
+    uint16_t* pos_of = stage16 + IPT * NT;                        // second half of the staging buffer
+#pragma unroll
+    for (int r = 0; r < IPT; r++) {
+        const int pos = tid * IPT + r;
+        const uint32_t id = w[r] & 0xffffu;
+        stage16[pos] = (uint16_t)id;
+        if (pos < n) pos_of[id] = (uint16_t)pos;
+    }
+    __syncthreads();
+    for (int j = tid; j < n; j += NT) {
+        const uint32_t id = stage16[j];
+        sids[base + j] = (int32_t)(off + id);
+        if (lids) lids[base + j] = (uint16_t)id;
+        if (inv) inv[base + j] = pos_of[j];
+    }
+}
+
+template <int NT, int IPT, int WPS>
+static int launch_radix1w(const float* d_keys, const SegGeom& g, int num_indices, float* d_skeys,
+                          int32_t* d_sids, uint16_t* d_inv, uint16_t* d_lids, hipStream_t s) {
+    const size_t lds = (size_t)(IPT * NT + 64) * 4;
+    static DeviceOnce once;
+    {
+        const int rc = once.run([lds]() -> int {
+            DCIH_HIP(hipFuncSetAttribute((const void*)segsort_radix1w_kernel<NT, IPT, WPS>,
+                                         hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds));
+            return 0;
+        });
+        if (rc) return rc;
+    }
+    const int64_t blocks = (int64_t)num_indices * g.B;
+    if (blocks > 0x7fffffffLL) return fail(-1, "segsort: too many slices for one launch");
+    hipLaunchKernelGGL((segsort_radix1w_kernel<NT, IPT, WPS>), dim3((unsigned)blocks), dim3(NT), lds, s,
+                       d_keys, g, d_skeys, d_sids, d_inv, d_lids);
+    DCIH_HIP(hipGetLastError());
+    return 0;
+}
+
 // Merge path: how many elements of A are among the first d outputs of merging A
 // (la elements) with B (lb elements), A winning ties (its positions are smaller).
 // One wavefront searches 64 split points per round.
@@ -537,6 +724,9 @@ int segsort(const float* d_keys, int64_t key_stride, int num_indices, int64_t n,
 #define DCIH_RADIX(NT, IPT) \
     if (g.ppb <= (int64_t)(NT) * (IPT))  \
         return launch_radix<NT, IPT>(d_keys, g, num_indices, d_skeys, d_sids, d_inv, d_lids, nullptr, s)
+        // slices of 15 k to 19968 points: the one-word kernel, two workgroups per CU
+        if (g.ppb > 15000 && g.ppb <= 512 * 39)
+            return launch_radix1w<512, 39, 4>(d_keys, g, num_indices, d_skeys, d_sids, d_inv, d_lids, s);
         DCIH_RADIX(64, 9); DCIH_RADIX(64, 17); DCIH_RADIX(64, 25); DCIH_RADIX(64, 33);
         DCIH_RADIX(128, 21); DCIH_RADIX(128, 27); DCIH_RADIX(128, 33);
         DCIH_RADIX(256, 21); DCIH_RADIX(256, 27); DCIH_RADIX(256, 33); DCIH_RADIX(256, 39); DCIH_RADIX(256, 45);
