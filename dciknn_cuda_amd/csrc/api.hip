@@ -131,7 +131,7 @@ struct dcih_index {
     float* d_stop_hint = nullptr;       // [3][block_size] epoch-size hints learnt from earlier queries
     int hint_k = 0, hint_outer = 0, hint_T = 0, hint_maxc = 0;   // query shape the hints belong to
     int traversal = 0;                  // DCIH_OPT_TRAVERSAL value
-    int dense_min_promos = 384;         // DCIH_OPT_DENSE_MIN_PROMOTIONS value
+    int dense_min_promos = 160;         // DCIH_OPT_DENSE_MIN_PROMOTIONS value
     int append_mode = 0;                // DCIH_OPT_APPEND value
     unsigned long long* d_phase_ticks = nullptr;   // optional profile of the batch kernel
     // grow-only workspace: query scratch, and the unsorted keys during a build
