@@ -25,7 +25,7 @@ def _shape(rng):
     k = int(min(n, rng.choice([1, 3, 10, 40])))
     outer = int(rng.choice([0, 1, 2, 7, 40, 100000]))
     max_cand = int(rng.choice([1, k, 10 * k, 10 ** 6]))
-    dim = int(rng.choice([1, 2, 5, 16, 33]))
+    dim = int(rng.choice([1, 2, 4, 5, 16, 33, 64, 100, 128]))
     kind = str(rng.choice(["normal", "dup", "grid", "far"]))
     return M, L, n, B, T, k, outer, max_cand, dim, kind
 
