@@ -317,6 +317,12 @@ def main():
     # 16-bit ids, 16-bit inverse positions), per query its row, the rows of its candidates and
     # its per-partition result lists
     hbm_bytes = 8.0 * I * N + nq * (4.0 * dim + 4.0 * dim * C + 8.0 * min(k, ppb) * cfg["bs"])
+    hbm_model = ("index slices once (8 B per entry) + per query its row, %.0f candidate rows of %d B and "
+                 "its per-partition result lists" % (C, 4 * dim))
+    if kernel.startswith("exact_dists"):
+        # direct ranking: the rows once, per (query, point) a distance written, sorted and read back
+        hbm_bytes = 4.0 * N * dim + nq * (4.0 * dim + 12.0 * N + 8.0 * k)
+        hbm_model = "rows once + per (query, point) a 4-byte distance out and 8 bytes through the sort"
     hbm_gbs = hbm_bytes / (launch_ms * 1e-3) / 1e9
     valu_ops = MIN_INSTR_PER_ENTRY * float(own[0]) * nq
     valu_gops = valu_ops / (launch_ms * 1e-3) / 1e9
@@ -328,8 +334,7 @@ def main():
     else:
         roofline = dict(bound="hbm", kernel=kernel, achieved=hbm_gbs, peak=HBM_PEAK_GBS,
                         unit="GB/s", frac=hbm_gbs / HBM_PEAK_GBS,
-                        model="index slices once (8 B per entry) + per query its row, %.0f candidate "
-                              "rows of %d B and its per-partition result lists" % (C, 4 * dim))
+                        model=hbm_model)
     roofline.update(avg_launch_ms=launch_ms, hbm_bytes_per_launch=hbm_bytes, hbm_gbs=hbm_gbs,
                     hbm_frac=hbm_gbs / HBM_PEAK_GBS, valu_min_lane_instr_per_launch=valu_ops,
                     valu_frac=valu_gops / VALU_PEAK_GOPS,
