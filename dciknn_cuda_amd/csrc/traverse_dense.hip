@@ -118,6 +118,9 @@ __device__ inline float group_row_sums(float (&v)[N], int s) {
     }
 }
 
+typedef uint16_t u16x2 __attribute__((ext_vector_type(2)));
+typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
+
 template <int IPT>
 __global__ __launch_bounds__(kDT, 2) void traverse_dense_kernel(QueryArgs a, DenseLayout y) {
     extern __shared__ __align__(16) unsigned char smem[];
@@ -145,8 +148,6 @@ __global__ __launch_bounds__(kDT, 2) void traverse_dense_kernel(QueryArgs a, Den
     const int wave = tid / kWave;
     const int I = a.M * a.L;
     const int T = a.T;
-    const uint32_t T_magic = a.T_magic;
-    auto div_T = [&](int d) { return T > 1 ? (int)__umulhi((uint32_t)d, T_magic) : d; };
     const int X = a.xcds;
     const int xcd = (int)(blockIdx.x % X);
     const int64_t g0 = blockIdx.x / X, G = gridDim.x / X;
@@ -212,11 +213,24 @@ __global__ __launch_bounds__(kDT, 2) void traverse_dense_kernel(QueryArgs a, Den
             // ---- layout of the composite's windows: per simple index its left stream, then
             // its right one; where the query lies above every key the single (ghost) right
             // window comes first, as dci_next_closest_proj orders it (:264-265)
-            if (tid == 0) {
-                int at = 0;
-                for (int h = 0; h < a.L; h++) {
-                    const int i = m * a.L + h, p = s_p[i];
-                    const int nl = stream_windows(n, T, p, 0), nr = stream_windows(n, T, p, 1);
+            // (one lane per simple index, the first wavefront: L <= 64)
+            if (wave == 0) {
+                const int h = lane;
+                int nl = 0, nr = 0, p = 0;
+                if (h < a.L) {
+                    p = s_p[m * a.L + h];
+                    nl = stream_windows(n, T, p, 0);
+                    nr = stream_windows(n, T, p, 1);
+                }
+                int incl = nl + nr;
+#pragma unroll
+                for (int o = 1; o < kWave; o <<= 1) {
+                    const int t2 = __shfl_up(incl, o, kWave);
+                    if (lane >= o) incl += t2;
+                }
+                const int at = incl - (nl + nr);
+                if (h < a.L) {
+                    const int i = m * a.L + h;
                     const bool corner = p == n - 1 && T >= 2;
                     // In the table the index's windows lie by the positions they cover: left
                     // window j at place nl - 1 - j, right window j at nl + j; a position pos
@@ -226,17 +240,20 @@ __global__ __launch_bounds__(kDT, 2) void traverse_dense_kernel(QueryArgs a, Den
                     s_shift[i] = nl * T - p - 1;
                     const int w_left = at + nl - 1, w_right = at + nl;
                     if (corner) {
-                        s_seg[2 * h] = at; s_segstream[2 * h] = 2 * h + 1; s_segw[2 * h] = w_right; at += nr;
-                        s_seg[2 * h + 1] = at; s_segstream[2 * h + 1] = 2 * h; s_segw[2 * h + 1] = w_left; at += nl;
+                        s_seg[2 * h] = at; s_segstream[2 * h] = 2 * h + 1; s_segw[2 * h] = w_right;
+                        s_seg[2 * h + 1] = at + nr; s_segstream[2 * h + 1] = 2 * h; s_segw[2 * h + 1] = w_left;
                     } else {
-                        s_seg[2 * h] = at; s_segstream[2 * h] = 2 * h; s_segw[2 * h] = w_left; at += nl;
-                        s_seg[2 * h + 1] = at; s_segstream[2 * h + 1] = 2 * h + 1; s_segw[2 * h + 1] = w_right; at += nr;
+                        s_seg[2 * h] = at; s_segstream[2 * h] = 2 * h; s_segw[2 * h] = w_left;
+                        s_seg[2 * h + 1] = at + nl; s_segstream[2 * h + 1] = 2 * h + 1; s_segw[2 * h + 1] = w_right;
                     }
                 }
-                s_seg[2 * a.L] = at;
-                misc[dWin] = (uint32_t)at;
-                if (at > kDT * IPT || at >= 0x7fff) misc[dFail] = 1;
-                misc[dOr] = 0; misc[dAnd] = 0xffffffffu;
+                const int total = __shfl(incl, a.L - 1, kWave);
+                if (lane == 0) {
+                    s_seg[2 * a.L] = total;
+                    misc[dWin] = (uint32_t)total;
+                    if (total > kDT * IPT || total >= 0x7fff) misc[dFail] = 1;
+                    misc[dOr] = 0; misc[dAnd] = 0xffffffffu;
+                }
             }
             __syncthreads();
             if (misc[dFail]) break;
@@ -298,54 +315,173 @@ __global__ __launch_bounds__(kDT, 2) void traverse_dense_kernel(QueryArgs a, Den
             __syncthreads();
             phase(2);
             // the step of every window: its place in the sorted order (the first W sorted items
-            // are the windows), stored doubled so that the lane-0 flag fits beside it
+            // are the windows), stored doubled with bit 0 set: a lookup subtracts one where the
+            // point is not the window's first lane, which leaves the lane-0 flag beside the step
 #pragma unroll
             for (int r = 0; r < IPT; r++) {
                 const int sp = tid * IPT + r;
-                if (sp < W) rank16[rp[r] & 0xffffu] = (uint16_t)(sp << 1);
+                if (sp < W) rank16[rp[r] & 0xffffu] = (uint16_t)((sp << 1) | 1);
             }
             __syncthreads();
 
             // ---- every point: the latest of the steps of its L windows ------------------
-            // (sixteen points per thread at a time and four simple indices at once, so that
-            //  sixty-four reads of the inverse permutation are in flight per lane: the phase is
-            //  a chain of memory round trips and this makes it a short one)
-            constexpr int kP = 16, kH = 4;
+            // A thread takes eight consecutive points at a time: their positions in one simple
+            // index are one 16-byte read of the inverse permutation (slices start on 2-byte
+            // boundaries; the reads need no more).  The reads for two simple indices make a
+            // group, and the reads of three groups are in flight while one group is looked up
+            // (the rows read for distances by the CU's other workgroup keep the memory system
+            // busy: a read takes microseconds).  The last chunk of a slice is moved back to end at the
+            // slice's end: some points are then looked up twice, with the same result.  The
+            // phase is bound by vector-ALU issue, so the lookups are kept branch-free and short:
+            // for a power-of-two T two points at a time in packed 16-bit arithmetic, otherwise
+            // with 24-bit multiplies (32-bit ones run at a quarter of the rate).
             const uint16_t* invm = a.inv + (int64_t)m * a.L * a.N + off;
-            for (int c0 = 0; c0 < n; c0 += kDT * kP) {
-                uint32_t best[kP];         // step << 1 | lane-0 flag of the latest window so far
-#pragma unroll
-                for (int u = 0; u < kP; u++) best[u] = 0u;
-                for (int h0 = 0; h0 < a.L; h0 += kH) {
-                    int posv[kH][kP];
-#pragma unroll
-                    for (int hh = 0; hh < kH; hh++) {
-                        const uint16_t* invh = invm + (int64_t)min(h0 + hh, a.L - 1) * a.N;
-#pragma unroll
-                        for (int u = 0; u < kP; u++) posv[hh][u] = (int)invh[min(c0 + u * kDT + tid, n - 1)];
+            auto store_time = [&](int pt, uint32_t b) __attribute__((always_inline)) {
+                const uint32_t old = s_time[pt];      // ties: the earlier composite stays
+                if ((b >> 1) < (old >> 1)) s_time[pt] = (uint16_t)b;
+            };
+            if (n < 8) {
+                for (int pt = tid; pt < n; pt += kDT) {
+                    uint32_t best = 0u;
+                    for (int h = 0; h < a.L; h++) {
+                        const int i = m * a.L + h;
+                        const uint32_t x = (uint32_t)invm[(int64_t)h * a.N + pt] + (uint32_t)s_shift[i];
+                        const uint32_t w = T > 1 ? __umulhi(x, a.T_magic) : x;
+                        best = max(best, (uint32_t)rank16[s_tabbase[i] + w] - (x - w * (uint32_t)T != 0u ? 1u : 0u));
                     }
+                    store_time(pt, best);
+                }
+            } else {
+                auto run = [&](auto path_tag) __attribute__((always_inline)) {
+                    constexpr int kPath = decltype(path_tag)::value;     // 0: T = 2^s, s >= 1; 1: any T >= 2; 2: T = 1
+                    constexpr int kH = 2, kD = 4, kChunk = kDT * 8;
+                    const int ngrp = (a.L + kH - 1) / kH;
+                    const int NG = ((n + kChunk - 1) / kChunk) * ngrp;
+                    const unsigned char* tab0 = reinterpret_cast<const unsigned char*>(rank16);
+                    // path 0
+                    const uint32_t sm1 = (uint32_t)floor_log2(T > 1 ? T : 2) - 1u;
+                    const u16x2 sm1_pk = {(uint16_t)sm1, (uint16_t)sm1};
+                    const u16x2 mask_pk = {(uint16_t)(T - 1), (uint16_t)(T - 1)};
+                    const u16x2 one_pk = {1, 1};
+                    // path 1: d / T for 0 <= d < 65536 is the upper 32 bits of (d << q_sh) *
+                    // ceil(2^(32 - q_sh) / T); rounding the factor up adds less than 1 / T to d / T,
+                    // which never reaches the next integer; q_sh = 8 serves 2 <= T <= 256, q_sh = 0
+                    // the wider windows, and both factors stay below 2^24 either way.
+                    const uint32_t q_sh = T <= 256 ? 8u : 0u;
+                    const uint32_t q_magic = T > 1 ? (uint32_t)(((1ull << (32 - q_sh)) + (uint32_t)T - 1) / (uint32_t)T) : 0u;
+                    const uint32_t q_T = (uint32_t)T << q_sh;
+                    uint32_t best[kPath == 0 ? 4 : 8];     // path 0: two points a word
+                    auto chunk_start = [&](int c0) { return min(c0 + 8 * tid, n - 8); };
+                    auto issue = [&](int c0, int h0, u32x4 (&pv)[kH]) __attribute__((always_inline)) {
 #pragma unroll
-                    for (int hh = 0; hh < kH; hh++) {
-                        if (h0 + hh >= a.L) break;
-                        const int i = m * a.L + h0 + hh;
-                        const int shift = s_shift[i];
-                        const uint16_t* tab = rank16 + s_tabbase[i];
+                        for (int hh = 0; hh < kH; hh++) {
+                            const uint16_t* invh = invm + (int64_t)min(h0 + hh, a.L - 1) * a.N;
+                            __builtin_memcpy(&pv[hh], invh + (uint32_t)chunk_start(c0), 16);
+                        }
+                    };
+                    auto consume = [&](int c0, int h0, const u32x4 (&pv)[kH]) __attribute__((always_inline)) {
+                        if (h0 == 0) {
 #pragma unroll
-                        for (int u = 0; u < kP; u++) {
-                            const int x = posv[hh][u] + shift, w = div_T(x);
-                            const uint32_t v = (uint32_t)tab[w] | (x - w * T == 0 ? 1u : 0u);
-                            best[u] = max(best[u], v);      // (steps differ from window to window)
+                            for (int e = 0; e < (kPath == 0 ? 4 : 8); e++) best[e] = 0u;
+                        }
+                        // every table read of the group is issued before the first is used
+                        uint32_t tv[kH][8];
+                        u16x2 rem[kH][4];
+#pragma unroll
+                        for (int hh = 0; hh < kH; hh++) {
+                            const int i = m * a.L + min(h0 + hh, a.L - 1);   // (past L: the last index again)
+                            const uint32_t shift = (uint32_t)s_shift[i];
+                            const unsigned char* tab = tab0 + 2 * s_tabbase[i];
+                            const uint32_t wd[4] = {pv[hh].x, pv[hh].y, pv[hh].z, pv[hh].w};
+#pragma unroll
+                            for (int j = 0; j < 4; j++) {
+                                if constexpr (kPath == 0) {
+                                    const u16x2 shift_pk = {(uint16_t)shift, (uint16_t)shift};
+                                    const u16x2 x = __builtin_bit_cast(u16x2, wd[j]) + shift_pk;
+                                    // twice the window's place: the byte offset of its table entry
+                                    const uint32_t w2 = __builtin_bit_cast(uint32_t, x >> sm1_pk) & 0xfffefffeu;
+                                    // (spelled out: the compiler's own form of min(r, 1) is
+                                    //  two compares, two selects and a byte permute)
+                                    asm("v_pk_min_u16 %0, %1, %2" : "=v"(rem[hh][j]) : "v"(x & mask_pk), "v"(one_pk));
+                                    tv[hh][2 * j] = *reinterpret_cast<const uint16_t*>(tab + (w2 & 0xffffu));
+                                    tv[hh][2 * j + 1] = *reinterpret_cast<const uint16_t*>(tab + (w2 >> 16));
+                                } else {
+#pragma unroll
+                                    for (int e = 0; e < 2; e++) {
+                                        const uint32_t pos = e ? wd[j] >> 16 : wd[j] & 0xffffu;
+                                        if constexpr (kPath == 1) {
+                                            const uint32_t xs = (pos << q_sh) + (shift << q_sh);
+                                            uint32_t w;
+                                            asm("v_mul_hi_u32_u24 %0, %1, %2" : "=v"(w) : "s"(q_magic), "v"(xs));
+                                            tv[hh][2 * j + e] = *reinterpret_cast<const uint16_t*>(tab + 2 * w);
+                                            const uint32_t off_lane = (uint32_t)(__umul24(w, q_T) != xs);
+                                            if (e) rem[hh][j].y = (uint16_t)off_lane; else rem[hh][j].x = (uint16_t)off_lane;
+                                        } else {
+                                            tv[hh][2 * j + e] = *reinterpret_cast<const uint16_t*>(tab + 2 * (pos + shift));
+                                        }
+                                    }
+                                }
+                            }
+                        }
+#pragma unroll
+                        for (int hh = 0; hh < kH; hh++)
+#pragma unroll
+                            for (int j = 0; j < 4; j++) {
+                                if constexpr (kPath == 0) {
+                                    const u16x2 val =
+                                        __builtin_bit_cast(u16x2, tv[hh][2 * j] | (tv[hh][2 * j + 1] << 16)) - rem[hh][j];
+                                    best[j] = __builtin_bit_cast(uint32_t,
+                                        __builtin_elementwise_max(__builtin_bit_cast(u16x2, best[j]), val));
+                                } else if constexpr (kPath == 1) {
+                                    best[2 * j] = max(best[2 * j], tv[hh][2 * j] - (uint32_t)rem[hh][j].x);
+                                    best[2 * j + 1] = max(best[2 * j + 1], tv[hh][2 * j + 1] - (uint32_t)rem[hh][j].y);
+                                } else {
+                                    best[2 * j] = max(best[2 * j], tv[hh][2 * j]);
+                                    best[2 * j + 1] = max(best[2 * j + 1], tv[hh][2 * j + 1]);
+                                }
+                            }
+                        if (h0 + kH >= a.L) {
+                            // (read, choose, write back unconditionally: a point that two threads
+                            //  hold, at the moved-back end of a slice, gets the same value from both)
+                            const int pt0 = chunk_start(c0);
+                            uint32_t old[8];
+#pragma unroll
+                            for (int e = 0; e < 8; e++) old[e] = s_time[pt0 + e];
+#pragma unroll
+                            for (int e = 0; e < 8; e++) {
+                                uint32_t b;
+                                if constexpr (kPath == 0) b = (best[e >> 1] >> ((e & 1) * 16)) & 0xffffu;
+                                else b = best[e];
+                                // ties: the earlier composite stays
+                                s_time[pt0 + e] = (uint16_t)((b >> 1) < (old[e] >> 1) ? b : old[e]);
+                            }
+                        }
+                    };
+                    // A ring of kD groups: the reads of the next kD - 1 groups are in flight while
+                    // one group is looked up.  The loop body has no branch (the counters of reads
+                    // under way are only exact in straight-line code): past the last group the reads
+                    // repeat the slice's last chunk and the lookups change nothing that is stored.
+                    int cc = 0, hc = 0, ci = 0, hi = 0;     // (chunk base, first simple index) of the group to consume / to issue
+                    auto advance = [&](int& c, int& h) { h += kH; if (h >= a.L) { h = 0; c += kChunk; } };
+                    u32x4 pv[kD][kH];
+#pragma unroll
+                    for (int d = 0; d < kD; d++) {
+                        issue(ci, hi, pv[d]);
+                        advance(ci, hi);
+                    }
+                    for (int g = 0; g < NG; g += kD) {
+#pragma unroll
+                        for (int d = 0; d < kD; d++) {
+                            consume(cc, hc, pv[d]);
+                            advance(cc, hc);
+                            issue(ci, hi, pv[d]);
+                            advance(ci, hi);
                         }
                     }
-                }
-#pragma unroll
-                for (int u = 0; u < kP; u++) {
-                    const int pt = c0 + u * kDT + tid;
-                    if (pt < n) {
-                        const uint32_t old = s_time[pt];      // ties: the earlier composite stays
-                        if ((best[u] >> 1) < (old >> 1)) s_time[pt] = (uint16_t)best[u];
-                    }
-                }
+                };
+                if (T > 1 && (T & (T - 1)) == 0) run(std::integral_constant<int, 0>{});
+                else if (T > 1) run(std::integral_constant<int, 1>{});
+                else run(std::integral_constant<int, 2>{});
             }
             __syncthreads();
             phase(3);

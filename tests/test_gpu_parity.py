@@ -183,6 +183,7 @@ CASES = [
     (30000, 16, 16, 2, 15, 16, 4, 50, 300, "normal"),       # L = 15, several hundred promotions per partition
     (20000, 16, 16, 3, 8, 4, 16, 100, 40, "normal"),        # three composites, k = 100
     (6000, 16, 12, 2, 6, 3, 2, 5, 10_000, "normal"),        # narrow windows, stop by c0 >= 10k
+    (9000, 16, 16, 2, 4, 2, 300, 10, 3, "normal"),          # T > 256
 ]
 
 
