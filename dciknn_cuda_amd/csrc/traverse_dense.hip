@@ -265,27 +265,47 @@ __global__ __launch_bounds__(kDT, 2) void traverse_dense_kernel(QueryArgs a, Den
             {
                 int seg = 0;
                 const int first = tid * IPT;
-                while (seg < 2 * a.L - 1 && s_seg[seg + 1] <= first) seg++;
-                int seg_end = s_seg[seg + 1];
-                int sidx = s_segstream[seg];
-                int seg_at = s_seg[seg];
-                int seg_w = s_segw[seg];
+                {   // the first segment that ends behind `first` (empty segments are skipped)
+                    int lo = 0, hi = 2 * a.L - 1;
+                    while (lo < hi) {
+                        const int mid = (lo + hi) >> 1;
+                        if (s_seg[mid + 1] <= first) lo = mid + 1; else hi = mid;
+                    }
+                    seg = lo;
+                }
                 // (offsets from the composite's first slice; all reads are issued before any is used)
                 const float* kbase = a.skeys + (int64_t)m * a.L * a.N + off;
                 uint32_t koff[IPT];
                 float qv[IPT];
+                // Per segment: where its windows' keys lie and which way they run.  Window j of
+                // a right stream starts at position p + 1 + j * T and takes table place
+                // seg_w + j; of a left stream, p - T + 1 - j * T and seg_w - j; the key read is
+                // the one at that position moved into the slice.
+                int seg_end, pos_cur, pos_step, w_cur, w_step;
+                uint32_t h_base;
+                float q_seg;
+                auto enter = [&](int idx) {
+                    seg_end = s_seg[seg + 1];
+                    const int sidx = s_segstream[seg], j = idx - s_seg[seg], h = sidx >> 1;
+                    const int p = s_p[m * a.L + h];
+                    q_seg = s_qp[m * a.L + h];
+                    h_base = (uint32_t)h * (uint32_t)a.N;
+                    if (sidx & 1) { pos_step = T; pos_cur = p + 1 + j * T; w_step = 1; w_cur = s_segw[seg] + j; }
+                    else { pos_step = -T; pos_cur = p - T + 1 - j * T; w_step = -1; w_cur = s_segw[seg] - j; }
+                };
+                enter(first);
 #pragma unroll
                 for (int r = 0; r < IPT; r++) {
                     const int idx = first + r;
-                    while (idx >= seg_end && seg < 2 * a.L - 1) {
-                        seg++;
-                        seg_end = s_seg[seg + 1]; sidx = s_segstream[seg]; seg_at = s_seg[seg]; seg_w = s_segw[seg];
+                    if (idx >= seg_end && seg < 2 * a.L - 1) {
+                        do { seg++; } while (seg < 2 * a.L - 1 && s_seg[seg + 1] <= idx);
+                        enter(idx);
                     }
-                    const int h = sidx >> 1, p = s_p[m * a.L + h], j = idx - seg_at;
-                    const int pos = (sidx & 1) ? min(p + 1 + j * T, n - 1) : max(p - T + 1 - j * T, 0);
-                    koff[r] = (uint32_t)h * (uint32_t)a.N + (uint32_t)(idx < W ? pos : 0);
-                    qv[r] = s_qp[m * a.L + h];
-                    rp[r] = (uint32_t)(idx < W ? ((sidx & 1) ? seg_w + j : seg_w - j) : 0);    // the sort's payload: the window's place in the table
+                    koff[r] = h_base + (uint32_t)(idx < W ? min(max(pos_cur, 0), n - 1) : 0);
+                    qv[r] = q_seg;
+                    rp[r] = (uint32_t)(idx < W ? w_cur : 0);    // the sort's payload: the window's place in the table
+                    pos_cur += pos_step;
+                    w_cur += w_step;
                 }
                 float kv[IPT];
 #pragma unroll
