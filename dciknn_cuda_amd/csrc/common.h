@@ -120,48 +120,43 @@ __device__ inline void wave_row_dists(const float* const (&rows)[R], const float
 #pragma unroll
     for (int r = 0; r < R; r++) dist[r] = sqrtf(wave_sum(acc[r]));
 }
-// The same sums in the same order for 16-byte aligned rows, with U consecutive 16-byte
-// pieces of each of the R rows in flight per lane (long rows: more bytes under way per
-// wavefront while the adds stay in sequence).
+// The same sums in the same order for 16-byte aligned rows of at least 256
+// elements, with no lane condition around a read: U pieces (256 elements apart) of each of
+// the R rows are read at once by every lane; a lane whose piece would begin past the row's
+// end reads the row's first piece again and adds nothing.  (Rows whose length is no multiple
+// of 256 elements otherwise end in an extra round of reads by a few lanes.)
 template <int R, int U>
-__device__ inline void wave_row_dists_deep(const float* const (&rows)[R], const float* q, int dim,
+__device__ inline void wave_row_dists_wide(const float* const (&rows)[R], const float* q, int dim,
                                            float (&dist)[R]) {
     typedef float v4f __attribute__((ext_vector_type(4)));
     const int lane = lane_id();
     float acc[R];
 #pragma unroll
     for (int r = 0; r < R; r++) acc[r] = 0.f;
-    int j = lane * 4;
-    for (; j + (U - 1) * kWave * 4 < dim; j += U * kWave * 4) {
+    for (int j0 = 0; j0 < dim; j0 += U * kWave * 4) {
         v4f x[U][R];
-#pragma unroll
-        for (int u = 0; u < U; u++)
-#pragma unroll
-            for (int r = 0; r < R; r++) x[u][r] = *reinterpret_cast<const v4f*>(rows[r] + j + u * kWave * 4);
+        int jc[U];
+        bool ok[U];
 #pragma unroll
         for (int u = 0; u < U; u++) {
-            const int ju = j + u * kWave * 4;
-            const float q0 = q[ju], q1 = q[ju + 1], q2 = q[ju + 2], q3 = q[ju + 3];
+            const int ju = j0 + u * kWave * 4 + lane * 4;
+            ok[u] = ju < dim;
+            jc[u] = ok[u] ? ju : lane * 4;
+#pragma unroll
+            for (int r = 0; r < R; r++) x[u][r] = *reinterpret_cast<const v4f*>(rows[r] + jc[u]);
+        }
+#pragma unroll
+        for (int u = 0; u < U; u++) {
+            const float q0 = q[jc[u]], q1 = q[jc[u] + 1], q2 = q[jc[u] + 2], q3 = q[jc[u] + 3];
 #pragma unroll
             for (int r = 0; r < R; r++) {
-                float d = x[u][r].x - q0; acc[r] = __builtin_fmaf(d, d, acc[r]);
-                d = x[u][r].y - q1; acc[r] = __builtin_fmaf(d, d, acc[r]);
-                d = x[u][r].z - q2; acc[r] = __builtin_fmaf(d, d, acc[r]);
-                d = x[u][r].w - q3; acc[r] = __builtin_fmaf(d, d, acc[r]);
+                float s2 = acc[r];
+                float d = x[u][r].x - q0; s2 = __builtin_fmaf(d, d, s2);
+                d = x[u][r].y - q1; s2 = __builtin_fmaf(d, d, s2);
+                d = x[u][r].z - q2; s2 = __builtin_fmaf(d, d, s2);
+                d = x[u][r].w - q3; s2 = __builtin_fmaf(d, d, s2);
+                acc[r] = ok[u] ? s2 : acc[r];
             }
-        }
-    }
-    for (; j < dim; j += kWave * 4) {
-        v4f x[R];
-#pragma unroll
-        for (int r = 0; r < R; r++) x[r] = *reinterpret_cast<const v4f*>(rows[r] + j);
-        const float q0 = q[j], q1 = q[j + 1], q2 = q[j + 2], q3 = q[j + 3];
-#pragma unroll
-        for (int r = 0; r < R; r++) {
-            float d = x[r].x - q0; acc[r] = __builtin_fmaf(d, d, acc[r]);
-            d = x[r].y - q1; acc[r] = __builtin_fmaf(d, d, acc[r]);
-            d = x[r].z - q2; acc[r] = __builtin_fmaf(d, d, acc[r]);
-            d = x[r].w - q3; acc[r] = __builtin_fmaf(d, d, acc[r]);
         }
     }
 #pragma unroll

@@ -648,7 +648,7 @@ __global__ __launch_bounds__(kDT, 2) void traverse_dense_kernel(QueryArgs a, Den
                         for (int r = 0; r < R; r++) rows[r] = a.data + (off + pts[r]) * a.dim;
                         float d[R];
                         const float* const (&crows)[R] = rows;
-                        if (R > 2) wave_row_dists_deep<R, 2>(crows, s_q, a.dim, d);      // (only chosen for aligned rows)
+                        if (R > 2) wave_row_dists_wide<R, 16 / R>(crows, s_q, a.dim, d);  // (only chosen for aligned rows of 512 elements or more)
                         else wave_row_dists<R>(crows, s_q, a.dim, vec4, d);
 #pragma unroll
                         for (int r = 0; r < R; r++)
@@ -747,7 +747,9 @@ __global__ __launch_bounds__(kDT, 2) void traverse_dense_kernel(QueryArgs a, Den
             using std::integral_constant;
             if (y.tiles && vec4 && a.dim <= 64 && y.quota >= kWave) run_tiles(integral_constant<int, 16>{});
             else if (y.tiles && vec4 && a.dim <= 128 && y.quota >= kWave) run_tiles(integral_constant<int, 32>{});
-            else if (vec4 && !a.blind && a.dim >= 512 && y.quota >= 8) run_rounds(integral_constant<int, 64>{}, integral_constant<int, 8>{});
+            // long rows: sixteen 16-byte reads in flight per lane, as whole 1 KiB pieces of as few rows as hold them
+            else if (vec4 && !a.blind && a.dim == 512 && y.quota >= 8) run_rounds(integral_constant<int, 64>{}, integral_constant<int, 8>{});
+            else if (vec4 && !a.blind && a.dim > 512 && y.quota >= 4) run_rounds(integral_constant<int, 64>{}, integral_constant<int, 4>{});
             else run_rounds(integral_constant<int, 64>{}, integral_constant<int, 2>{});
         }
         if (lane == 0) atomicAdd(&misc[dCand], ncand);

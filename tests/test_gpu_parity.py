@@ -184,6 +184,8 @@ CASES = [
     (20000, 16, 16, 3, 8, 4, 16, 100, 40, "normal"),        # three composites, k = 100
     (6000, 16, 12, 2, 6, 3, 2, 5, 10_000, "normal"),        # narrow windows, stop by c0 >= 10k
     (9000, 16, 16, 2, 4, 2, 300, 10, 3, "normal"),          # T > 256
+    (3000, 8, 512, 2, 4, 3, 16, 10, 5, "normal"),           # long rows: two 1 KiB pieces
+    (3000, 8, 1100, 2, 4, 3, 16, 10, 5, "normal"),          # long rows: five pieces, the last one short
 ]
 
 
