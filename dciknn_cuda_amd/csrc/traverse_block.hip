@@ -177,6 +177,10 @@ __global__ __launch_bounds__(NT, MINW) void traverse_block_kernel(QueryArgs a, B
     // traversal itself has gone that far.  Which kernel finishes an item never shows in
     // the results.
     const bool may_hand_over = a.dense_items != nullptr && a.dense_min_promos > 0;
+    // An item that is already under way here is worth moving only from twice the number of
+    // promotions at which a whole call is routed to the dense kernel: below that, finishing
+    // it here is cheaper than starting over there.
+    const int64_t hand_over_at = 2 * (int64_t)a.dense_min_promos;
     auto hand_to_dense = [&]() {
         if (threadIdx.x == 0) {
             const int x = (int)(blockIdx.x % a.xcds);
@@ -184,7 +188,7 @@ __global__ __launch_bounds__(NT, MINW) void traverse_block_kernel(QueryArgs a, B
             a.dense_items[(int64_t)x * a.dense_cap + sl] = (int32_t)item;
         }
     };
-    if (may_hand_over && a.stop_hint && a.stop_hint[a.B + b] >= (float)a.dense_min_promos) {
+    if (may_hand_over && a.stop_hint && a.stop_hint[a.B + b] >= (float)hand_over_at) {
         hand_to_dense();
         return;
     }
@@ -868,7 +872,7 @@ __global__ __launch_bounds__(NT, MINW) void traverse_block_kernel(QueryArgs a, B
         }
         phase(7);
         if (stop) break;
-        if (may_hand_over && misc[kNumCand] + misc[kEventCount] >= (uint32_t)a.dense_min_promos) {
+        if (may_hand_over && misc[kNumCand] + misc[kEventCount] >= (uint32_t)hand_over_at) {
             // (the stop hints still learn from it: the dense kernel records its stops too)
             hand_to_dense();
             return;

@@ -60,7 +60,7 @@ struct DenseLayout {
 constexpr int kWlist = 2 * kWave;        // candidates a wavefront keeps listed
 
 int dense_ipt_for(int64_t windows) {
-    for (int ipt : {9, 17, 25, 33})
+    for (int ipt : {9, 17, 25, 33, 41})
         if (windows <= (int64_t)kDT * ipt) return ipt;
     return 0;
 }
@@ -823,7 +823,8 @@ int query_dense_items(const QueryArgs& a_in, hipStream_t s) {
     if (y.ipt == 9) DCIH_DENSE(9);
     else if (y.ipt == 17) DCIH_DENSE(17);
     else if (y.ipt == 25) DCIH_DENSE(25);
-    else DCIH_DENSE(33);
+    else if (y.ipt == 33) DCIH_DENSE(33);
+    else DCIH_DENSE(41);
 #undef DCIH_DENSE
     DCIH_HIP(hipGetLastError());
     return 0;

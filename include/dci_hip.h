@@ -65,7 +65,9 @@ enum {
  * inside its last epoch, the dense kernel looks at every entry) and
  * DCIH_CTR_PROBES their own key reads.  DCIH_OPT_DENSE_MIN_PROMOTIONS: under
  * automatic choice, the number of promotions per (query, partition) from which
- * an item goes to the dense kernel (default 160; 0 = never).
+ * the dense kernel is used (default 160; 0 = never): a call whose stop rule needs
+ * that many (num_neighbours * thread_size) goes there as a whole, and the batch
+ * kernel hands over single items that reach twice that many.
  * DCIH_OPT_FORGET_HINTS (value ignored): drops what earlier queries taught the
  * handle about where traversals stop (used only to size the batch kernel's
  * epochs, never visible in results), so that the next call runs like a first one.

@@ -184,6 +184,7 @@ CASES = [
     (20000, 16, 16, 3, 8, 4, 16, 100, 40, "normal"),        # three composites, k = 100
     (6000, 16, 12, 2, 6, 3, 2, 5, 10_000, "normal"),        # narrow windows, stop by c0 >= 10k
     (9000, 16, 16, 2, 4, 2, 300, 10, 3, "normal"),          # T > 256
+    (40000, 16, 24, 2, 12, 4, 12, 10, 200, "normal"),       # 10032 windows per composite: the largest dense tables
     (3000, 8, 512, 2, 4, 3, 16, 10, 5, "normal"),           # long rows: two 1 KiB pieces
     (3000, 8, 1100, 2, 4, 3, 16, 10, 5, "normal"),          # long rows: five pieces, the last one short
 ]
@@ -192,7 +193,7 @@ CASES = [
 def _dense_fits(n, M, L, B, T, k):
     ppb = -(-n // B)
     return (M <= 64 and L <= 64 and ppb <= 32766 and min(k, ppb) <= 512 and
-            L * (ppb // T + 3) <= 33 * 256)
+            L * (ppb // T + 3) <= 41 * 256)
 
 
 @pytest.mark.parametrize("traversal", ["step", "batch", "dense", "auto"])

@@ -52,7 +52,7 @@ def dense_fits(n, M, L, B, T, k):
     """Shapes the dense traversal kernel's tables take (it refuses the others)."""
     ppb = -(-n // B)
     return (M <= 64 and L <= 64 and ppb <= 32766 and min(k, ppb) <= 512 and
-            L * (ppb // T + 3) <= 33 * 256)
+            L * (ppb // T + 3) <= 41 * 256)
 
 
 def batch_fits(n, M, L, B, k):
