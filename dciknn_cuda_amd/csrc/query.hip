@@ -16,6 +16,8 @@
 // workgroup slice of global scratch.  A window of T sorted entries is visited
 // by T lanes at once (in 64-lane slabs when T > 64); promoted points are found
 // with a ballot and their rows are read by the whole wavefront.
+#include <math.h>
+
 #include "common.h"
 #include "kernels.h"
 
@@ -381,9 +383,16 @@ int query(const QueryArgs& a_in, hipStream_t s, hipEvent_t* ev, bool* ran) {
     // Left to choose: the stop rule needs k promotions by a window's first lane, which takes
     // about k * T promotions in all; from the number at which the dense kernel is the cheaper
     // one, every item goes straight to it (no hints needed: also a first call is routed right).
-    if (a.mode == 0 && can_dense && !a.blind && a.dense_min_promos > 0 &&
-        (int64_t)a.k_stop * a.T >= (int64_t)a.dense_min_promos)
-        a.mode = 3;
+    // The step limit can ask for more: a traversal that must consume the fraction f of a
+    // composite's windows before it may stop has by then promoted about f^L of the partition
+    // (a point needs all L of its windows; nearby windows come first, so this is on the low
+    // side), unless max_candidates first-lane promotions end it earlier.
+    if (a.mode == 0 && can_dense && !a.blind && a.dense_min_promos > 0) {
+        const double windows = (double)a.L * ((double)a.ppb / (double)a.T);
+        const double f = fmin(1.0, (double)a.stop_at / fmax(1.0, windows));
+        const double by_steps = fmin((double)a.ppb * pow(f, (double)a.L), (double)a.max_cand * (double)a.T);
+        if (fmax((double)a.k_stop * (double)a.T, by_steps) >= (double)a.dense_min_promos) a.mode = 3;
+    }
     const bool use_block = a.mode != 1 && a.mode != 3 && can_block;
     // the batch kernel hands items that need many promotions to the dense kernel
     if (!(use_block && a.mode == 0 && can_dense && a.dense_items && a.dense_min_promos > 0)) {
