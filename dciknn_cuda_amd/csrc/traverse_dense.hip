@@ -122,7 +122,7 @@ typedef uint16_t u16x2 __attribute__((ext_vector_type(2)));
 typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
 
 template <int IPT>
-__global__ __launch_bounds__(kDT, 2) void traverse_dense_kernel(QueryArgs a, DenseLayout y) {
+__global__ __launch_bounds__(kDT, (IPT <= 9 ? 3 : 2)) void traverse_dense_kernel(QueryArgs a, DenseLayout y) {
     extern __shared__ __align__(16) unsigned char smem[];
     uint32_t* misc = reinterpret_cast<uint32_t*>(smem);
     uint32_t* scan_tmp = misc + dMiscWords;                           // 64 words
@@ -328,21 +328,53 @@ __global__ __launch_bounds__(kDT, 2) void traverse_dense_kernel(QueryArgs a, Den
             }
             __syncthreads();
             phase(1);
-            // (the pads need no pass of their own: they start behind every window, every
-            //  digit of theirs is the largest, and the passes are stable)
-            const uint32_t varying = misc[dOr] ^ misc[dAnd];
-            lds_radix_passes<kDT, IPT>(k, rp, stage, stage + IPT * kDT, scan_tmp, varying);
-            __syncthreads();
-            phase(2);
-            // the step of every window: its place in the sorted order (the first W sorted items
-            // are the windows), stored doubled with bit 0 set: a lookup subtracts one where the
-            // point is not the window's first lane, which leaves the lane-0 flag beside the step
+            // the step of every window: its place in the sorted order, stored doubled with bit 0
+            // set: a lookup subtracts one where the point is not the window's first lane, which
+            // leaves the lane-0 flag beside the step
+            bool sorted_small = false;
+            if constexpr (IPT == 9) {
+                // Up to 1024 windows (short partitions): a bitonic sort held in registers of
+                // (priority, layout index, table place) words — the layout index makes equal
+                // priorities keep their order, as the stable radix passes do — takes a few
+                // microseconds where eight radix passes over 2304 slots take thirty.
+                if (W <= 1024) {
+                    sorted_small = true;
+                    const int np = W <= 256 ? 256 : (W <= 512 ? 512 : 1024);
+                    unsigned long long* s64 = reinterpret_cast<unsigned long long*>(stage);
 #pragma unroll
-            for (int r = 0; r < IPT; r++) {
-                const int sp = tid * IPT + r;
-                if (sp < W) rank16[rp[r] & 0xffffu] = (uint16_t)((sp << 1) | 1);
+                    for (int r = 0; r < IPT; r++) {
+                        const int idx = tid * IPT + r;
+                        if (idx < np)
+                            s64[idx] = idx < W ? ((unsigned long long)k[r] << 32) | ((unsigned long long)idx << 16) | (rp[r] & 0xffffu)
+                                               : ~0ull;
+                    }
+                    bitonic_sort_u64_by256(s64, np);
+                    unsigned long long mine[4];
+                    const int per = np / kDT;
+#pragma unroll
+                    for (int e = 0; e < 4; e++) mine[e] = e < per ? s64[tid * per + e] : ~0ull;
+                    __syncthreads();                    // the table takes the sorted words' room
+#pragma unroll
+                    for (int e = 0; e < 4; e++) {
+                        const int sp = tid * per + e;
+                        if (e < per && sp < W) rank16[(uint32_t)mine[e] & 0xffffu] = (uint16_t)((sp << 1) | 1);
+                    }
+                }
+            }
+            if (!sorted_small) {
+                // (the pads need no pass of their own: they start behind every window, every
+                //  digit of theirs is the largest, and the passes are stable)
+                const uint32_t varying = misc[dOr] ^ misc[dAnd];
+                lds_radix_passes<kDT, IPT>(k, rp, stage, stage + IPT * kDT, scan_tmp, varying);
+                __syncthreads();
+#pragma unroll
+                for (int r = 0; r < IPT; r++) {
+                    const int sp = tid * IPT + r;
+                    if (sp < W) rank16[rp[r] & 0xffffu] = (uint16_t)((sp << 1) | 1);      // (the first W sorted items are the windows)
+                }
             }
             __syncthreads();
+            phase(2);
 
             // ---- every point: the latest of the steps of its L windows ------------------
             // A thread takes eight consecutive points at a time: their positions in one simple
