@@ -133,7 +133,7 @@ __global__ __launch_bounds__(kRadixThreads, (kRadixThreads == 256 && IPT > 45) ?
     uint32_t* misc = rs + IPT * kRadixThreads + 8 * kRadixThreads;   // 64 words
 
     const int tid = threadIdx.x;
-    const int lane = tid & 63, wave = tid >> 6;
+    const int lane = tid & 63;
     // packed == null: the workgroup sorts a whole slice and writes the final arrays;
     // else it sorts one tile of a slice into packed (key, position in slice) words
     // for the merge passes

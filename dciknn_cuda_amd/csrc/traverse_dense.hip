@@ -466,7 +466,7 @@ __global__ __launch_bounds__(kDT, (IPT <= 9 ? 3 : 2)) void traverse_dense_kernel
                                             uint32_t w;
                                             asm("v_mul_hi_u32_u24 %0, %1, %2" : "=v"(w) : "s"(q_magic), "v"(xs));
                                             tv[hh][2 * j + e] = *reinterpret_cast<const uint16_t*>(tab + 2 * w);
-                                            const uint32_t off_lane = (uint32_t)(__umul24(w, q_T) != xs);
+                                            const uint32_t off_lane = (uint32_t)((uint32_t)__umul24(w, q_T) != xs);
                                             if (e) rem[hh][j].y = (uint16_t)off_lane; else rem[hh][j].x = (uint16_t)off_lane;
                                         } else {
                                             tv[hh][2 * j + e] = *reinterpret_cast<const uint16_t*>(tab + 2 * (pos + shift));
