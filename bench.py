@@ -53,8 +53,8 @@ MIN_INSTR_PER_ENTRY = 4.0
 TUNED = {
     "c1": dict(bs=100, ts=10, outer=5000),
     "c2": dict(bs=56, ts=2, outer=500),
-    "c3": dict(bs=500, ts=32, outer=530),
-    "c4": dict(bs=100, ts=16, outer=500),
+    "c3": dict(bs=400, ts=128, outer=100),
+    "c4": dict(bs=100, ts=64, outer=126),
     "c5": dict(bs=1280, ts=64, outer=10),
 }
 RECALL_TARGET = {"c1": 0.95, "c2": 0.95, "c3": 0.9, "c4": 0.95, "c5": None}

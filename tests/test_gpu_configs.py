@@ -28,8 +28,8 @@ pytestmark = pytest.mark.gpu
 DIST_RTOL = 1e-5
 
 # the settings bench.py runs these configurations at (block_size, thread_size, outer)
-C3_SETTING = (500, 32, 530)
-C4_SETTING = (100, 16, 500)
+C3_SETTING = (400, 128, 100)
+C4_SETTING = (100, 64, 126)
 C5_SETTING = (1280, 64, 10)
 
 
@@ -113,7 +113,9 @@ def _kernels_agree(dci, Qd, k, outer, modes):
 @pytest.mark.parametrize("n,B,T,outer,modes", [
     # slices of 65000 points: the build sorts them as tiles + merge passes; near the batch kernel's limit
     (130_000, 2, 32, 1700, ["step", "batch", "auto"]),
-    # the full-size setting's partition length (20000) and step limit
+    # the full-size setting's partition length (25000) and windows: stops by c0 >= 100, ~12800 promotions
+    (75_000, 3, 128, 100, ["step", "dense", "auto"]),
+    # an earlier full-size setting: 20000-point partitions, stops by the step limit
     (60_000, 3, 32, 530, ["step", "batch", "dense", "auto"]),
     # narrow windows: stops by c0 >= k well before the step limit
     (60_000, 6, 1, 60, ["step", "batch", "dense", "auto"]),
@@ -132,7 +134,8 @@ def test_c3_reduced_against_oracle(gpu, oracle, n, B, T, outer, modes):
 
 
 @pytest.mark.parametrize("n,B,T,outer,modes", [
-    (30_000, 3, 16, 500, ["step", "batch", "dense", "auto"]),     # the full-size regime: step limit, ~1200 promotions per partition
+    (30_000, 3, 64, 126, ["step", "dense", "auto"]),              # the full-size setting: step limit, ~1300 promotions per partition
+    (30_000, 3, 16, 500, ["step", "batch", "dense", "auto"]),     # the same regime with narrower windows
     (30_000, 3, 10, 500, ["step", "batch", "dense", "auto"]),     # the reference example's thread_size
     (70_000, 2, 4, 2000, ["step", "batch", "auto"]),              # 35000-point slices
 ])
