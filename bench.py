@@ -55,7 +55,7 @@ TUNED = {
     "c2": dict(bs=56, ts=2, outer=500),
     "c3": dict(bs=400, ts=128, outer=100),
     "c4": dict(bs=100, ts=64, outer=126),
-    "c5": dict(bs=1280, ts=64, outer=10),
+    "c5": dict(bs=900, ts=128, outer=10),
 }
 RECALL_TARGET = {"c1": 0.95, "c2": 0.95, "c3": 0.9, "c4": 0.95, "c5": None}
 # queries per leg that would otherwise take minutes on the large workloads
