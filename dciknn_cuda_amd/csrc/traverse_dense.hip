@@ -121,8 +121,10 @@ __device__ inline float group_row_sums(float (&v)[N], int s) {
 typedef uint16_t u16x2 __attribute__((ext_vector_type(2)));
 typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
 
-template <int IPT>
-__global__ __launch_bounds__(kDT, (IPT <= 9 ? 3 : 2)) void traverse_dense_kernel(QueryArgs a, DenseLayout y) {
+// WPS = wavefronts per SIMD the register allocation leaves room for: three where the tables let
+// three workgroups share a CU's LDS, else two (and 256 registers instead of 168).
+template <int IPT, int WPS>
+__global__ __launch_bounds__(kDT, WPS) void traverse_dense_kernel(QueryArgs a, DenseLayout y) {
     extern __shared__ __align__(16) unsigned char smem[];
     uint32_t* misc = reinterpret_cast<uint32_t*>(smem);
     uint32_t* scan_tmp = misc + dMiscWords;                           // 64 words
@@ -841,22 +843,23 @@ int query_dense_items(const QueryArgs& a_in, hipStream_t s) {
                                                       : block_items(a.xcds, a.B, a.nq) / a.xcds;
     per_xcd = max((int64_t)1, min(per_xcd, most));
     const unsigned grid = (unsigned)(per_xcd * a.xcds);
-#define DCIH_DENSE(IPT)                                                                          \
+#define DCIH_DENSE(IPT, WPS)                                                                        \
     do {                                                                                         \
         static DeviceOnce once;                                                                  \
         const int rc_attr = once.run([]() -> int {                                               \
-            DCIH_HIP(hipFuncSetAttribute((const void*)traverse_dense_kernel<IPT>,                \
+            DCIH_HIP(hipFuncSetAttribute((const void*)traverse_dense_kernel<IPT, WPS>,             \
                                          hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024)); \
             return 0;                                                                            \
         });                                                                                      \
         if (rc_attr) return rc_attr;                                                             \
-        hipLaunchKernelGGL((traverse_dense_kernel<IPT>), dim3(grid), dim3(kDT), y.lds_bytes, s, a, y); \
+        hipLaunchKernelGGL((traverse_dense_kernel<IPT, WPS>), dim3(grid), dim3(kDT), y.lds_bytes, s, a, y); \
     } while (0)
-    if (y.ipt == 9) DCIH_DENSE(9);
-    else if (y.ipt == 17) DCIH_DENSE(17);
-    else if (y.ipt == 25) DCIH_DENSE(25);
-    else if (y.ipt == 33) DCIH_DENSE(33);
-    else DCIH_DENSE(41);
+    if (y.ipt == 9 && per_cu >= 3) DCIH_DENSE(9, 3);
+    else if (y.ipt == 9) DCIH_DENSE(9, 2);
+    else if (y.ipt == 17) DCIH_DENSE(17, 2);
+    else if (y.ipt == 25) DCIH_DENSE(25, 2);
+    else if (y.ipt == 33) DCIH_DENSE(33, 2);
+    else DCIH_DENSE(41, 2);
 #undef DCIH_DENSE
     DCIH_HIP(hipGetLastError());
     return 0;
