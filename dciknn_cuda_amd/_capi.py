@@ -1,4 +1,4 @@
-"""ctypes binding of libdci_hip.so (the C-ABI in include/dci_hip.h).
+"""ctypes binding of libdci_hip.so (the C-ABI in include/dci_hip.h and include/dci_hip_debug.h).
 
 The library is the product: there is no fallback.  Importing this module
 without a built library raises; build it with `python -m dciknn_cuda_amd.build`.
@@ -21,7 +21,7 @@ NOALLOC_SCRATCH_BYTES = 32 << 20
 NUM_TIMERS = 7
 T_PROJECT, T_SEGSORT, T_QPROJECT, T_TRAVERSE, T_MERGE, T_BATCH, T_DENSE = range(7)
 
-# name -> (restype, argtypes); one line per declaration in include/dci_hip.h
+# name -> (restype, argtypes); one line per declaration in include/dci_hip.h and include/dci_hip_debug.h
 _c = ctypes
 SIGNATURES = {
     "dcih_last_error": (_c.c_char_p, []),

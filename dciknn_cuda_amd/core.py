@@ -9,7 +9,9 @@ counters, kernel choice) goes to the C-ABI directly.  Additions, all keyword-onl
 optional: `seed` / `directions` at construction and the `directions` property
 (the reference can neither seed, inject nor read its directions), and
 `return_int` / `return_counters` on `query`, and `traversal` / `set_traversal`
-to pick the query kernel.
+to pick the query kernel.  One deliberate difference: an index of more than
+2**24 + 1 points refuses to return ids as float32 (they would be rounded) and
+asks for `return_int=True`.
 """
 import torch
 
@@ -19,6 +21,20 @@ from . import _dci_cuda as _ext   # built by `python -m dciknn_cuda_amd.build`; 
 
 def _stream_ptr(device):
     return torch.cuda.current_stream(device).cuda_stream
+
+
+# float32 holds every integer up to 2**24 exactly and none of the odd ones above
+_MAX_FLOAT_ID = 1 << 24
+
+
+def _refuse_rounded_ids(num_points):
+    """The reference returns ids as float32 (src/dci_cuda.cpp:111), which rounds ids
+    above 2**24 to a neighbouring point's.  An index that large answers only with
+    integer ids."""
+    if num_points > _MAX_FLOAT_ID + 1:
+        raise ValueError(
+            "this index holds %d points and float32 ids are exact only up to %d: "
+            "pass return_int=True to query() to get int32 ids" % (num_points, _MAX_FLOAT_ID))
 
 
 class DCI(object):
@@ -156,6 +172,8 @@ class DCI(object):
             raise ValueError("num_neighbours exceeds the number of indexed points")
         max_num_candidates = 10 * num_neighbours
         nq = _query.shape[0]
+        if not return_int:
+            _refuse_rounded_ids(self.num_points)
         if not return_int and not return_counters:
             # the reference's own route: one flat float tensor, ids first (core.py:90-92)
             _query_result = _ext._dci_query(self._capsule, self._dim, nq, _query.flatten(),
@@ -233,6 +251,7 @@ class MDCI(object):
         _query = _query.detach().clone().to(self.dcis[0]._device)
         d0 = self.dcis[0]
         d0._check_data(_query)
+        _refuse_rounded_ids(d0.num_points)
         max_num_candidates = 10 * num_neighbours
         res = _ext._dci_multi_query([dc._capsule for dc in self.dcis], d0._dim, _query.shape[0],
                                     [_query.flatten()], num_neighbours, blind, num_outer_iterations,

@@ -1,4 +1,5 @@
-// Host side of libdci_hip.so: the C-ABI declared in include/dci_hip.h.
+// Host side of libdci_hip.so: the C-ABI declared in include/dci_hip.h (and the
+// inspection entry points of include/dci_hip_debug.h).
 //
 // Mirrors the host functions of the reference (dci_init, dci_add, dci_query,
 // dci_clear, dci_reset, dci_free: src/dci_cuda_kernel.cu:77-187, :777-899) but
@@ -13,6 +14,7 @@
 #include <vector>
 
 #include "../../include/dci_hip.h"
+#include "../../include/dci_hip_debug.h"
 #include "common.h"
 #include "kernels.h"
 
@@ -89,6 +91,7 @@ static __device__ __align__(256) unsigned char scratch[kScratchBytes];
 
 namespace {
 constexpr int kMaxDevices = 64;
+constexpr int kMaxXcds = 32;      // dies per device the query scratch has list lengths for (256 bytes: 1 + 32 words used)
 std::mutex g_scratch_mu;
 void* g_scratch_ptr[kMaxDevices] = {};
 
@@ -269,7 +272,7 @@ extern "C" {
 
 const char* dcih_last_error(void) { return g_last_error.c_str(); }
 
-int dcih_abi_version(void) { return 1; }
+int dcih_abi_version(void) { return 2; }
 
 int dcih_create(int dim, int num_comp_indices, int num_simp_indices, int device,
                 uint64_t seed, dcih_index** out) {
@@ -290,7 +293,10 @@ int dcih_create(int dim, int num_comp_indices, int num_simp_indices, int device,
     h->device = device; h->seed = seed;
     {   // dies with an L2 of their own: the batch traversal orders its work by them
         int xcds = 0;
-        if (hipDeviceGetAttribute(&xcds, hipDeviceAttributeNumberOfXccs, device) == hipSuccess && xcds >= 1)
+        // (the per-die list lengths of the query scratch have room for kMaxXcds dies; a device
+        //  that reports more, or none, is treated as one of 8)
+        if (hipDeviceGetAttribute(&xcds, hipDeviceAttributeNumberOfXccs, device) == hipSuccess &&
+            xcds >= 1 && xcds <= kMaxXcds)
             h->xcds = xcds;
         (void)hipGetLastError();
     }
@@ -419,6 +425,15 @@ int dcih_append(dcih_index* h, int dim, int64_t num_points, const float* d_data,
     float* ukeys = h->d_ukeys;
     int64_t cap = h->own_rows;
     int64_t have_keys = (h->n > 0 && h->d_data == h->d_own) ? std::min(h->ukeys_rows, h->n) : 0;
+    const int spare = 1 - h->cur;
+    // Merging the old slices with the sorted new points instead of sorting everything again.
+    // Both are built; left to choose, the append sorts: the one-pass LDS sort moves 16 bytes per
+    // index entry, split + merge + inverse move 40, and on an MI355X the sort is the faster of the
+    // two at every size of the incremental workload (8.7 against 9.0 ms for 1M onto 19M points).
+    const bool merge = h->n > 0 && h->append_mode == 2 && h->d_inv != nullptr &&
+                       segsort_append_supported(h->n, total, block_size);
+    if (h->append_mode == 2 && h->n > 0 && !merge)
+        return fail(DCIH_EUNSUPPORTED, "dcih_append: this shape cannot be appended by merging (partitions too long)");
     float* fresh_rows = nullptr;
     float* fresh_keys = nullptr;
     if (!rows || cap < total) {
@@ -432,15 +447,6 @@ int dcih_append(dcih_index* h, int dim, int64_t num_points, const float* d_data,
         rows = fresh_rows;
         ukeys = fresh_keys;
     }
-    const int spare = 1 - h->cur;
-    // Merging the old slices with the sorted new points instead of sorting everything again.
-    // Both are built; left to choose, the append sorts: the one-pass LDS sort moves 16 bytes per
-    // index entry, split + merge + inverse move 40, and on an MI355X the sort is the faster of the
-    // two at every size of the incremental workload (8.7 against 9.0 ms for 1M onto 19M points).
-    const bool merge = h->n > 0 && h->append_mode == 2 && h->d_inv != nullptr &&
-                       segsort_append_supported(h->n, total, block_size);
-    if (h->append_mode == 2 && h->n > 0 && !merge)
-        return fail(DCIH_EUNSUPPORTED, "dcih_append: this shape cannot be appended by merging (partitions too long)");
     const size_t tmp_bytes = merge ? segsort_append_tmp_bytes(I, total) : segsort_tmp_bytes(I, total, block_size);
     int rc = ensure_arena(h, h->n > 0 ? spare : h->cur,
                           std::max(arena_layout(I, total, block_size).total,

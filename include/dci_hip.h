@@ -82,7 +82,12 @@ enum { DCIH_OPT_TRAVERSAL = 0, DCIH_OPT_DENSE_MIN_PROMOTIONS = 1, DCIH_OPT_FORGE
 /* Message for the last failing call on this thread ("" if none). */
 const char* dcih_last_error(void);
 
-/* Library/ABI version, bumped on any signature change. */
+/*
+ * Library/ABI version, bumped on any change a caller built against an older header
+ * could trip over.  2: dcih_last_timings writes DCIH_NUM_TIMERS = 7 values (5 in
+ * version 1), DCIH_OPT_TRAVERSAL accepts 3, DCIH_OPT_APPEND and dcih_query_noalloc
+ * exist, and the two inspection entry points moved to dci_hip_debug.h.
+ */
 int dcih_abi_version(void);
 
 /*
@@ -181,8 +186,14 @@ int dcih_query(dcih_index* h, int dim, int num_queries, const float* d_query,
 /*
  * dcih_query for callers that cannot allocate device memory: code under HIP graph
  * capture, tight serving loops, harnesses that forbid hipMalloc.  It has no
- * counterpart in the reference.  Same arguments, same results and same kernels as
- * dcih_query, but every byte of scratch (query projections, per-partition result
+ * counterpart in the reference.  Same arguments and same traversal kernels as
+ * dcih_query, and the same results bit for bit, with one exception: where
+ * dcih_query computes the answer directly because the stop rule provably cannot
+ * fire (see there; the reference's own example configuration is such a shape), this
+ * entry point still runs the traversal, whose distances are summed in a different
+ * order: the neighbour sets are then the same and the distances agree to 1e-5
+ * relative, not in every bit (and neighbours at tied distances may swap places).
+ * Every byte of scratch (query projections, per-partition result
  * lists, hand-over list between the two traversal kernels, global visit counters
  * of partitions too large for on-chip memory) comes from one array of
  * DCIH_NOALLOC_SCRATCH_BYTES that is part of the library's code object, so each
@@ -223,15 +234,6 @@ int dcih_set_option(dcih_index* h, int option, int value);
 int dcih_profile(dcih_index* h, int enable);
 int dcih_last_timings(dcih_index* h, float* h_ms);
 
-/*
- * Phase profile of the batch traversal kernel (no counterpart in the
- * reference).  d_ticks is NULL (off) or a zeroed device array of 16 uint64 that
- * later dcih_query calls add to: [0..7] = 100 MHz ticks one thread of every
- * workgroup spent in set-up, bound selection, range search, streaming, undo,
- * promotion ranking, replay, distances/top-k; [8] = epochs, [9] = workgroups.
- */
-int dcih_phase_profile(dcih_index* h, uint64_t* d_ticks);
-
 /* Number of points currently indexed (0 when empty). */
 int64_t dcih_num_points(const dcih_index* h);
 
@@ -268,18 +270,6 @@ int dcih_project(const float* d_dirs, int num_indices, const float* d_rows,
                  int64_t num_rows, int dim, float* d_out, void* stream);
 int dcih_segsort(const float* d_keys, int num_indices, int64_t num_points,
                  int block_size, float* d_skeys, int32_t* d_sids, void* stream);
-
-/*
- * Launch geometry of the batch traversal kernel (no counterpart in the reference;
- * pure host arithmetic, no GPU needed): with `xcds` dies, block_size partitions and
- * num_queries queries, returns the number of workgroups one launch starts, or -1
- * if the shape cannot be launched; if b and q are not NULL and 0 <= block < that
- * number, *b / *q receive the partition and query workgroup `block` works on, or
- * -1 / -1 if it has nothing to do.  *queries_per_launch (if not NULL) receives how
- * many queries one launch may cover (a launch is limited to 2^32 - 1 threads).
- */
-int64_t dcih_debug_launch_map(int xcds, int block_size, int num_queries, int64_t block,
-                              int* b, int* q, int* queries_per_launch);
 
 #ifdef __cplusplus
 }

@@ -1,5 +1,5 @@
 """Host-side checks that need no GPU: the C-ABI library loads and exports what
-include/dci_hip.h declares, argument errors come back as status codes, and the
+include/*.h declare, argument errors come back as status codes, and the
 Python front end validates its inputs like dciknn_cuda/core.py:53-92 does."""
 import ctypes
 import os
@@ -12,9 +12,12 @@ ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
 
 
 def _declared():
-    text = open(os.path.join(ROOT, "include", "dci_hip.h")).read()
-    text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
-    return sorted(set(re.findall(r"\b(dcih_[a-z_]+)\s*\(", text)))
+    names = set()
+    for header in ("dci_hip.h", "dci_hip_debug.h"):
+        text = open(os.path.join(ROOT, "include", header)).read()
+        text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
+        names |= set(re.findall(r"\b(dcih_[a-z_]+)\s*\(", text))
+    return sorted(names)
 
 
 def test_library_exports_every_declared_symbol():
@@ -26,7 +29,7 @@ def test_library_exports_every_declared_symbol():
         assert hasattr(lib, name), "libdci_hip.so lacks %s" % name
         assert name in _capi.SIGNATURES, "no ctypes signature for %s" % name
     assert set(_capi.SIGNATURES) == set(names)
-    assert _capi.lib().dcih_abi_version() == 1
+    assert _capi.lib().dcih_abi_version() == 2
 
 
 def test_null_and_bad_arguments_return_status_codes():
@@ -148,6 +151,27 @@ def test_freed_instance_raises():
         d.add(torch.zeros(2, 4))
     with pytest.raises(RuntimeError):
         d.query(torch.zeros(2, 4), 1)
+
+
+def test_float_ids_are_refused_where_they_would_be_rounded():
+    """float32 cannot hold ids above 2**24: the default (float) result is refused there,
+    before any device work, and return_int=True is the way through."""
+    from dciknn_cuda_amd import core
+
+    class FakeCuda(torch.Tensor):
+        @property
+        def is_cuda(self):
+            return True
+
+    d = _bare(4)
+    d._dci_inst = object()
+    q = torch.zeros(2, 4).as_subclass(FakeCuda)
+    d.num_points = (1 << 24) + 2
+    with pytest.raises(ValueError, match="return_int=True"):
+        d.query(q, 3)
+    core._refuse_rounded_ids((1 << 24) + 1)      # ids 0 .. 2**24 are all exact
+    with pytest.raises(ValueError):
+        core._refuse_rounded_ids(20_000_000)
 
 
 def test_mdci_accepts_one_device_only():
