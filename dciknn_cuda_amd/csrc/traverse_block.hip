@@ -19,18 +19,24 @@
 //    c0(kk) >= k and (kk+1 >= outer*L or c0(kk) >= max_candidates), where c0
 //    counts promotions whose last window held the point in lane 0 (:598-607).
 //
-// An epoch picks a priority bound per composite index, finds by binary search
-// how many windows of every stream lie below it, and lets all lanes stream the
-// new index ranges (coalesced 4-byte id reads, packed LDS visit counters).  A
-// counter reaching L is a promotion; only for those few points the exact step
-// is computed: the inverse permutation gives the point's position in each of
-// the L simple indices, the farthest of its windows is the last one visited,
-// and that window's rank is a sum of 2L binary searches.  Promotions are then
-// replayed in (step, composite) order to apply the stop rule.  An epoch that
-// promotes too many points at once is undone (the same ranges are streamed
-// again, subtracting) and retried smaller.  Whatever does not fit the fixed LDS
-// tables is handed to the step-by-step kernel through a redo list, so results
-// never depend on which kernel produced them.
+// An epoch picks a priority bound per composite index and finds by binary search
+// how many windows of every stream lie below it.  The windows a simple index has
+// consumed cover one run of positions [lo, hi) of its sorted slice, so the points
+// composite m has visited in all of its L simple indices are those whose position
+// lies inside the run in every one of them: all lanes scan the inverse permutation
+// (the position of every point in every slice, 16 bits each, eight points per
+// 16-byte read) and test run membership two points per instruction in packed
+// 16-bit arithmetic.  Only for the few points found the exact step is computed:
+// the farthest of the point's L windows is the last one visited, and that
+// window's rank is a sum of 2L binary searches.  Promotions are then replayed in
+// (step, composite) order to apply the stop rule.  An epoch that promotes too
+// many points at once is dropped and retried smaller.  Whatever does not fit the
+// fixed LDS tables is handed to the step-by-step kernel through a redo list, so
+// results never depend on which kernel produced them.
+#include <stdlib.h>
+
+#include <type_traits>
+
 #include "common.h"
 #include "kernels.h"
 #include "traverse_common.h"
@@ -41,22 +47,22 @@ namespace {
 
 constexpr int kMaxEpochs = 100000;
 
-enum Misc {   // 32-bit scalars shared by the workgroup; kStreamedLo must stay 8-byte aligned
+enum Misc {   // 32-bit scalars shared by the workgroup
     kPromoCount = 0, kEventCount, kAccCount, kFail, kStop, kC0, kStopStepLo, kStopStepHi,
-    kArmedLo, kArmedHi, kStreamedLo, kStreamedHi, kArmed, kNumCand, kTopN, kProbes, kMiscWords
+    kArmedLo, kArmedHi, kScannedLo, kScannedHi, kArmed, kNumCand, kTopN, kProbes, kMiscWords
 };
 
 struct BlockLayout {
-    int cbits, wpc, seen_words, mark_words, counter_words;
-    int off_idx;      // per simple index: p, qp            (2 * I words)
-    int off_stream;   // per stream: consumed, previous, total, range lo/hi, chunks, pos0, prefix (10 * 2I + 1 words, incl. stride and composite number)
-    int off_chunk0;   // per stream: global index of its first 16-byte chunk (2I 64-bit words)
-    int off_comp;     // per composite: rho bits, K, active, previous K, sum of inverse priorities (5 * M words)
+    int seen_words;   // one bit per point of the partition
+    int flag_words;   // seen bits + per composite the points it has promoted: (M + 1) * seen_words
+    int off_idx;      // per simple index: p, qp, and the visited run as packed 16-bit pairs (4 * I words)
+    int off_stream;   // per stream: consumed, previous, total, stride, composite number (5 * 2I words)
+    int off_comp;     // per composite: rho bits, K, active, previous K, sum of inverse priorities, scan flag (6 * M words)
     int off_q;        // query row
     int off_samp;     // per stream: 16 sampled window priorities of the current epoch's range
-    int off_promo, off_events, off_acc, off_sort, off_cnt;
+    int off_promo, off_events, off_acc, off_sort, off_flags;
     int promo_cap;    // promotions one epoch may produce (table size)
-    int promo_max;    // above this an epoch is undone and halved
+    int promo_max;    // above this an epoch is dropped and halved
     int event_cap;    // promotions waiting for the other composites (= accepted candidates per replay)
     int sort_cap;     // power of two >= kcap + 128: top-k plus one batch of candidates
     size_t lds_bytes;
@@ -65,20 +71,12 @@ struct BlockLayout {
 BlockLayout make_block_layout(const QueryArgs& a) {
     BlockLayout y;
     const int I = a.M * a.L;
-    y.cbits = counter_bits_of(a.L);
-    const int64_t fpw = 32 / y.cbits;
-    y.wpc = (int)((a.ppb + fpw - 1) / fpw);
     y.seen_words = (int)((a.ppb + 31) / 32);
-    // promoted points are marked by the all-ones counter value; where L itself is that
-    // value (15, 255) a bitmap per composite marks them instead
-    y.mark_words = a.L == (1 << y.cbits) - 1 ? a.M * y.seen_words : 0;
-    y.counter_words = a.M * y.wpc + y.seen_words + y.mark_words;
+    y.flag_words = (a.M + 1) * y.seen_words;
     int o = kMiscWords * 4;
-    y.off_idx = o;      o += 2 * I * 4;
-    y.off_stream = o;   o += (10 * 2 * I + 2) * 4;
-    o = (o + 7) & ~7;
-    y.off_chunk0 = o;   o += 2 * I * 8;
-    y.off_comp = o;     o += 5 * a.M * 4;
+    y.off_idx = o;      o += 4 * I * 4;
+    y.off_stream = o;   o += 5 * 2 * I * 4;
+    y.off_comp = o;     o += 6 * a.M * 4;
     y.off_q = o;        o += ((a.dim + 3) & ~3) * 4;
     // small tables keep more workgroups resident per CU; an item that overflows them
     // is redone by the step-by-step kernel
@@ -100,38 +98,32 @@ BlockLayout make_block_layout(const QueryArgs& a) {
     o = (o + 15) & ~15;
     y.off_events = o;   o += y.event_cap * 8;
     y.off_sort = o;     o += y.sort_cap * 8;
-    y.off_cnt = o;
-    y.lds_bytes = (size_t)o + (size_t)y.counter_words * 4;
+    y.off_flags = o;
+    y.lds_bytes = (size_t)o + (size_t)y.flag_words * 4;
     return y;
 }
 
 // MINW = waves per SIMD the register allocation must leave room for: LDS decides how
 // many workgroups fit a CU, and the kernel should not be the tighter limit.
-template <int NT, int CBITS, int MINW>
+template <int NT, int MINW>
 __global__ __launch_bounds__(NT, MINW) void traverse_block_kernel(QueryArgs a, BlockLayout y) {
-    constexpr uint32_t kFpw = 32 / CBITS;                       // counters per 32-bit word
-    constexpr int kFshift = CBITS == 4 ? 3 : 2;                 // log2(kFpw)
-    constexpr uint32_t kCmask = (1u << CBITS) - 1u;
     extern __shared__ __align__(16) unsigned char smem[];
     uint32_t* misc = reinterpret_cast<uint32_t*>(smem);
     int* s_p = reinterpret_cast<int*>(smem + y.off_idx);
     float* s_qp = reinterpret_cast<float*>(s_p + a.M * a.L);
+    uint32_t* s_lo2 = reinterpret_cast<uint32_t*>(s_qp + a.M * a.L);  // first position of the visited run, twice
+    uint32_t* s_lm2 = s_lo2 + a.M * a.L;                              // its length - 1, twice
     int* s_c = reinterpret_cast<int*>(smem + y.off_stream);          // windows consumed
     int* s_cprev = s_c + 2 * a.M * a.L;                               // ... at epoch start
     int* s_ns = s_cprev + 2 * a.M * a.L;                              // windows in the stream
-    int* s_ra = s_ns + 2 * a.M * a.L;                                 // epoch's position range [ra, rb)
-    int* s_rb = s_ra + 2 * a.M * a.L;
-    int* s_nch = s_rb + 2 * a.M * a.L;                                // 16-byte chunks the range touches
-    int* s_pos0 = s_nch + 2 * a.M * a.L;                              // position of the first chunk's first id
-    int* s_stride = s_pos0 + 2 * a.M * a.L;                           // windows to try next epoch
+    int* s_stride = s_ns + 2 * a.M * a.L;                             // windows to try next epoch
     int* s_mof = s_stride + 2 * a.M * a.L;                            // composite the stream belongs to
-    int* s_pref = s_mof + 2 * a.M * a.L;                              // whole-chunk prefix sums (2I + 1)
-    long long* s_chunk0 = reinterpret_cast<long long*>(smem + y.off_chunk0);
     uint32_t* s_rho = reinterpret_cast<uint32_t*>(smem + y.off_comp); // per composite
     uint32_t* s_K = s_rho + a.M;
     uint32_t* s_active = s_K + a.M;
     uint32_t* s_Kprev = s_active + a.M;
     float* s_hsum = reinterpret_cast<float*>(s_Kprev + a.M);
+    uint32_t* s_noscan = reinterpret_cast<uint32_t*>(s_hsum + a.M);   // some simple index of the composite has visited nothing yet
     float* s_q = reinterpret_cast<float*>(smem + y.off_q);
     uint32_t* s_samp = reinterpret_cast<uint32_t*>(smem + y.off_samp);
     uint32_t* promo = reinterpret_cast<uint32_t*>(smem + y.off_promo);
@@ -139,13 +131,20 @@ __global__ __launch_bounds__(NT, MINW) void traverse_block_kernel(QueryArgs a, B
     uint32_t* acc_step = acc + y.event_cap;       // blind querying only
     unsigned long long* events = reinterpret_cast<unsigned long long*>(smem + y.off_events);
     unsigned long long* sortbuf = reinterpret_cast<unsigned long long*>(smem + y.off_sort);
-    uint32_t* cnt = reinterpret_cast<uint32_t*>(smem + y.off_cnt);
-    uint32_t* seen = cnt + (size_t)a.M * y.wpc;
-    uint32_t* marked = seen + y.seen_words;          // only where y.mark_words > 0
+    uint32_t* seen = reinterpret_cast<uint32_t*>(smem + y.off_flags);
+    uint32_t* marked = seen + y.seen_words;          // [M][seen_words]: promoted under composite m in an accepted epoch
 
-    const int tid = threadIdx.x;
-    const int lane = tid & (kWave - 1);
-    const int wave = tid / kWave;
+    // The thread numbers are made opaque again at the start of every phase (fresh_thread_ids):
+    // otherwise the compiler computes each phase's lane groupings and per-thread addresses once,
+    // before the epoch loop, and keeps them all in registers (or scratch) across every phase.
+    int tid = threadIdx.x;
+    int lane = tid & (kWave - 1);
+    int wave = tid / kWave;
+    auto fresh_thread_ids = [&]() {
+        asm volatile("" : "+v"(tid));
+        lane = tid & (kWave - 1);
+        wave = tid / kWave;
+    };
     constexpr int kWaves = NT / kWave;
     // optional phase profile: thread 0 adds the 100 MHz ticks each phase took
     unsigned long long tick = a.phase_ticks ? wall_clock64() : 0ull;
@@ -199,7 +198,7 @@ __global__ __launch_bounds__(NT, MINW) void traverse_block_kernel(QueryArgs a, B
     auto div_T = [&](int d) { return T > 1 ? (int)__umulhi((uint32_t)d, T_magic) : d; };
 
     // ---- set-up ---------------------------------------------------------------
-    for (int w = tid; w < y.counter_words; w += NT) cnt[w] = 0;
+    for (int w = tid; w < y.flag_words; w += NT) seen[w] = 0;
     for (int j = tid; j < a.dim; j += NT) s_q[j] = a.query[(int64_t)qi * a.dim + j];
     if (tid < kMiscWords) misc[tid] = 0;
     uint32_t probes = 0;
@@ -256,7 +255,7 @@ __global__ __launch_bounds__(NT, MINW) void traverse_block_kernel(QueryArgs a, B
         if (tid < a.M) s_Kprev[tid] = 0;
     }
     __syncthreads();
-    phase(0);
+    phase(0); if (a.dense_cap < 0 && -a.dense_cap == 0 + 1) return; fresh_thread_ids();
 
     auto load_stream = [&](int s) {
         Stream st;
@@ -266,42 +265,92 @@ __global__ __launch_bounds__(NT, MINW) void traverse_block_kernel(QueryArgs a, B
         return st;
     };
 
-    // Adds (or, for undo, removes) the visits of windows [cprev, c) of all streams.
-    // The loop is bound by vector-ALU issue, so it reads partition-relative 16-bit
-    // ids, eight per aligned 16-byte chunk, and keeps per-visit work to shift /
-    // mask / one LDS atomic without return value, with compile-time field widths;
-    // which counters reached L is found afterwards by one scan of the counter
-    // words (collect_promotions).  The whole-chunk interior of every stream's
-    // range is laid end to end: consecutive threads read consecutive chunks
-    // whatever stream they belong to, the next batch of reads in flight while the
-    // current one is counted.  The one or two partial chunks at the ends of a
-    // range are handled separately with masks.  Returns the entries streamed (same
-    // value on every thread).
-    auto visit = [&](uint32_t* __restrict__ mcnt, uint32_t local, bool undo) {
-        const uint32_t sh = (local & (kFpw - 1u)) * CBITS;
-        if (undo) atomicSub(&mcnt[local >> kFshift], 1u << sh);
-        else atomicAdd(&mcnt[local >> kFshift], 1u << sh);
-    };
-    // Counters that stand at exactly L belong to points promoted in this epoch:
-    // a point is visited once per simple index, so its counter never passes L, and
-    // promotions of earlier epochs were moved to the all-ones value (or, where L is
-    // that value, entered in a bitmap) when their epoch was accepted (mark_promotions).
-    auto collect_promotions = [&]() {
-        constexpr uint32_t kRep = CBITS == 4 ? 0x11111111u : 0x01010101u;
-        const uint32_t want = (uint32_t)a.L * kRep;
-        const int words = a.M * y.wpc;
-        for (int w = tid; w < words; w += NT) {
-            const uint32_t x = cnt[w] ^ want;                       // zero field <=> counter == L
-            if (((x - kRep) & ~x & (kRep << (CBITS - 1))) == 0u) continue;   // no zero field
-            const int m = w / y.wpc;
-            const uint32_t first = (uint32_t)(w - m * y.wpc) << kFshift;
+    // The points an epoch promotes.  The windows simple index i has consumed so far cover the
+    // positions [lo_i, hi_i) of its sorted slice (the left stream's windows end at the query
+    // position, the right stream's start there), so composite m has visited a point in all of
+    // its L simple indices exactly when the point's position lies in that run in every one of
+    // them.  Every thread takes eight consecutive points at a time: their positions in one
+    // simple index are ONE 16-byte read of the inverse permutation, and per pair of points
+    // membership costs three packed 16-bit instructions: pos - lo (wrapping), minus
+    // (length - 1) with unsigned saturation -- zero exactly when lo <= pos < hi -- and a
+    // running maximum over the simple indices, which ends at zero for the points inside all L
+    // runs.  Those not yet promoted under m in an earlier epoch (one bit per point and
+    // composite) go to the promotion list.  No state is left behind: an epoch that turns out
+    // too large is simply dropped.  The loop reads L * n positions per composite whatever the
+    // bound, four simple indices' reads in flight per thread.
+    typedef uint16_t u16x2 __attribute__((ext_vector_type(2)));
+    typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
+    typedef __attribute__((address_space(1))) const u32x4 g_u32x4;
+    // chunks of eight points start where the slices' reads are 16-byte aligned, if the slices of
+    // all simple indices can be aligned together (N a multiple of 8); else reads are unaligned
+    const int chunk_shift = (a.N & 7) == 0 ? (int)(off & 7) : 0;
+    const int nchunks = (n + chunk_shift + 7) >> 3;
+    auto scan_epoch = [&]() {
+        if (tid < a.M) s_noscan[tid] = 0;
+        __syncthreads();
+        if (tid < I) {
+            const int64_t p1 = (int64_t)s_p[tid] + 1;
+            const int lo = (int)max((int64_t)0, p1 - (int64_t)s_c[2 * tid] * T);
+            const int hi = (int)min((int64_t)n, p1 + (int64_t)s_c[2 * tid + 1] * T);
+            const uint32_t lm = (uint32_t)(hi - lo - 1) & 0xffffu;
+            s_lo2[tid] = ((uint32_t)lo & 0xffffu) * 0x10001u;
+            s_lm2[tid] = lm * 0x10001u;
+            if (hi <= lo) s_noscan[tid / a.L] = 1;
+        }
+        __syncthreads();
+        for (int m = 0; m < a.M; m++) {
+            if (s_noscan[m]) continue;
+            const uint16_t* inv_m = a.inv + (int64_t)m * a.L * a.N + off - chunk_shift;
+            const uint32_t* lo2 = s_lo2 + m * a.L;
+            const uint32_t* lm2 = s_lm2 + m * a.L;
+            const uint32_t* marked_m = marked + m * y.seen_words;
+            for (int c = tid; c < nchunks; c += NT) {
+                const int first = 8 * c - chunk_shift;      // partition-relative id of the chunk's first point
+                u16x2 worst[4];
 #pragma unroll
-            for (uint32_t f = 0; f < kFpw; f++) {
-                if (((x >> (f * CBITS)) & kCmask) == 0u) {
-                    if (y.mark_words > 0 &&
-                        ((marked[m * y.seen_words + ((first + f) >> 5)] >> ((first + f) & 31u)) & 1u)) continue;
+                for (int r = 0; r < 4; r++) worst[r] = u16x2{0, 0};
+                if (c == 0 || c == nchunks - 1) {            // places before the partition's first point or past its last
+#pragma unroll
+                    for (int r = 0; r < 4; r++) {
+                        const bool out0 = (uint32_t)(first + 2 * r) >= (uint32_t)n;
+                        const bool out1 = (uint32_t)(first + 2 * r + 1) >= (uint32_t)n;
+                        worst[r] = u16x2{(uint16_t)(out0 ? 0xffff : 0), (uint16_t)(out1 ? 0xffff : 0)};
+                    }
+                }
+                const uint16_t* at = inv_m + 8 * (int64_t)c;
+                auto group = [&](int h0, auto width) {
+                    constexpr int W = decltype(width)::value;
+                    u32x4 x[W];
+#pragma unroll
+                    for (int u = 0; u < W; u++) x[u] = *(g_u32x4*)(at + (int64_t)(h0 + u) * a.N);
+#pragma unroll
+                    for (int u = 0; u < W; u++) {
+                        const u16x2 lo = __builtin_bit_cast(u16x2, lo2[h0 + u]);
+                        const u16x2 lm = __builtin_bit_cast(u16x2, lm2[h0 + u]);
+                        const uint32_t w[4] = {x[u].x, x[u].y, x[u].z, x[u].w};
+#pragma unroll
+                        for (int r = 0; r < 4; r++) {
+                            const u16x2 d = __builtin_bit_cast(u16x2, w[r]) - lo;
+                            worst[r] = __builtin_elementwise_max(worst[r], __builtin_elementwise_sub_sat(d, lm));
+                        }
+                    }
+                };
+                int h0 = 0;
+                for (; h0 + 4 <= a.L; h0 += 4) group(h0, std::integral_constant<int, 4>());
+                if (h0 + 2 <= a.L) { group(h0, std::integral_constant<int, 2>()); h0 += 2; }
+                if (h0 < a.L) group(h0, std::integral_constant<int, 1>());
+                const u16x2 m01 = __builtin_elementwise_min(worst[0], worst[1]);
+                const u16x2 m23 = __builtin_elementwise_min(worst[2], worst[3]);
+                const uint32_t least = __builtin_bit_cast(uint32_t, __builtin_elementwise_min(m01, m23));
+                if (((least - 0x00010001u) & ~least & 0x80008000u) == 0u) continue;     // no 16-bit field is zero
+#pragma unroll
+                for (int e = 0; e < 8; e++) {
+                    const uint32_t w = __builtin_bit_cast(uint32_t, worst[e >> 1]);
+                    if (((w >> ((e & 1) * 16)) & 0xffffu) != 0u) continue;
+                    const uint32_t local = (uint32_t)(first + e);
+                    if ((marked_m[local >> 5] >> (local & 31u)) & 1u) continue;
                     const uint32_t slot = atomicAdd(&misc[kPromoCount], 1u);
-                    if (slot < (uint32_t)y.promo_cap) promo[slot] = (first + f) | ((uint32_t)m << 26);
+                    if (slot < (uint32_t)y.promo_cap) promo[slot] = local | ((uint32_t)m << 26);
                 }
             }
         }
@@ -309,158 +358,18 @@ __global__ __launch_bounds__(NT, MINW) void traverse_block_kernel(QueryArgs a, B
     auto mark_promotions = [&](uint32_t np) {
         for (uint32_t j = tid; j < np; j += NT) {
             const uint32_t local = promo[j] & 0x3ffffffu, m = promo[j] >> 26;
-            if (y.mark_words > 0) atomicOr(&marked[m * y.seen_words + (local >> 5)], 1u << (local & 31u));
-            else atomicOr(&cnt[(size_t)m * y.wpc + (local >> kFshift)], kCmask << ((local & (kFpw - 1u)) * CBITS));
+            atomicOr(&marked[m * y.seen_words + (local >> 5)], 1u << (local & 31u));
         }
     };
-    auto stream_epoch = [&](bool undo) {
-        constexpr int kUnroll = 4;
-        if (tid < S) {
-            const int i = tid >> 1;
-            int ra, rb;
-            stream_range(n, T, s_p[i], tid & 1, s_cprev[tid], s_c[tid], ra, rb);
-            s_ra[tid] = ra; s_rb[tid] = rb;
-            const int64_t base_idx = (int64_t)i * a.N + off;
-            const int64_t c_first = (base_idx + ra) >> 3;            // chunk holding position ra
-            const int64_t c_end = (base_idx + rb + 7) >> 3;          // one past the chunk holding rb-1
-            s_chunk0[tid] = c_first;
-            s_nch[tid] = rb > ra ? (int)(c_end - c_first) : 0;
-            s_pos0[tid] = (int)((c_first << 3) - base_idx);          // position of that chunk's first id
-        }
-        __syncthreads();
-        if (tid == 0) {          // prefix over the interior (whole) chunks of every stream
-            int acc_chunks = 0;
-            for (int s = 0; s < S; s++) {
-                s_pref[s] = acc_chunks;
-                acc_chunks += max(0, s_nch[s] - 2);
-            }
-            s_pref[S] = acc_chunks;
-        }
-        __syncthreads();
-        // (explicitly global: through a generic pointer the reads would also count as LDS
-        //  traffic and every wait on LDS would wait for them)
-        typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
-        typedef __attribute__((address_space(1))) const u32x4 g_u32x4;
-        typedef __attribute__((address_space(3))) uint32_t lds_u32;
-        g_u32x4* all = (g_u32x4*)a.lids;
-        // partial chunks: the first and the last chunk of every range
-        if (tid < 2 * S) {
-            const int s = tid >> 1;
-            const int nch = s_nch[s];
-            const int which = tid & 1;                 // 0 = first chunk, 1 = last chunk
-            if (nch > which) {
-                const int cidx = which ? nch - 1 : 0;
-                const u32x4 r = all[s_chunk0[s] + cidx];
-                const int pos0 = s_pos0[s] + (cidx << 3);
-                const int ra = s_ra[s], rb = s_rb[s];
-                const int m = (s >> 1) / a.L;
-                uint32_t* mcnt = cnt + (size_t)m * y.wpc;
-                const uint32_t w[4] = {r.x, r.y, r.z, r.w};
-#pragma unroll
-                for (int e = 0; e < 8; e++) {
-                    const int pos = pos0 + e;
-                    if (pos >= ra && pos < rb) visit(mcnt, (w[e >> 1] >> ((e & 1) * 16)) & 0xffffu, undo);
-                }
-            }
-        }
-        // whole chunks
-        const int total = s_pref[S];
-        // The stream a thread is in changes rarely: its description stays in registers and
-        // LDS is read only when a chunk number passes the end of the stream.  Addresses of
-        // a batch are all formed before its reads are issued, and the reads themselves are
-        // unconditional (a thread past the end re-reads the first chunk and ignores it), so
-        // they go out back to back.
-        auto counters_of = [&](int sidx) {      // LDS byte address of the stream's composite's counters
-            return (uint32_t)(uintptr_t)(lds_u32*)(cnt + (size_t)s_mof[sidx] * y.wpc);
-        };
-        int cur = 0, next_pref = s_pref[1];
-        uint32_t cbase = counters_of(0);
-        long long delta = s_chunk0[0] + 1 - s_pref[0];      // chunk number -> index into `all`
-        auto fetch = [&](int g0, u32x4 (&r)[kUnroll], uint32_t (&mr)[kUnroll]) {
-            g_u32x4* ptr[kUnroll];
-#pragma unroll
-            for (int u = 0; u < kUnroll; u++) {
-                const int g = g0 + u * NT + tid;
-                const int gg = min(g, total - 1);
-                while (gg >= next_pref) {
-                    cur++;
-                    next_pref = s_pref[cur + 1];
-                    cbase = counters_of(cur);
-                    delta = s_chunk0[cur] + 1 - s_pref[cur];
-                }
-                mr[u] = g < total ? cbase : 0u;          // 0: past the end, nothing to count
-                ptr[u] = all + (delta + gg);
-            }
-#pragma unroll
-            for (int u = 0; u < kUnroll; u++) r[u] = *ptr[u];
-        };
-        // Per visit four vector instructions and one atomic: a bit-field extract (or a
-        // shift, for the id in the upper half of a word) and a shift-add give the counter
-        // word's LDS address; the id scaled by the field width, taken modulo 32 by the
-        // shift instruction itself, is the field's bit offset.  The sequences are spelled
-        // out because the compiler's canonical form of the same arithmetic is longer.
-        constexpr uint32_t kCs = CBITS == 4 ? 2u : 3u;              // log2(CBITS)
-        const uint32_t field_scale = kCs;                            // SDWA operands cannot be literals
-        auto process = [&](const u32x4 (&r)[kUnroll], const uint32_t (&mr)[kUnroll]) {
-#pragma unroll
-            for (int u = 0; u < kUnroll; u++) {
-                if (mr[u] == 0u) continue;
-                const uint32_t base = mr[u];
-                const uint32_t w[4] = {r[u].x, r[u].y, r[u].z, r[u].w};
-#pragma unroll
-                for (int e = 0; e < 8; e++) {
-                    const uint32_t ww = w[e >> 1];
-                    uint32_t word, addr, bit;
-                    if (e & 1) {
-                        word = ww >> (16 + kFshift);
-                        asm("v_lshlrev_b32_sdwa %0, %1, %2 dst_sel:DWORD dst_unused:UNUSED_PAD "
-                            "src0_sel:DWORD src1_sel:WORD_1" : "=v"(bit) : "s"(field_scale), "v"(ww));
-                    } else {
-                        asm("v_bfe_u32 %0, %1, %2, %3" : "=v"(word) : "v"(ww), "n"(kFshift), "n"(16 - kFshift));
-                        bit = ww << kCs;
-                    }
-                    asm("v_lshl_add_u32 %0, %1, 2, %2" : "=v"(addr) : "v"(word), "v"(base));
-                    const uint32_t one = 1u << (bit & 31u);
-                    lds_u32* p = (lds_u32*)(uintptr_t)addr;
-                    if (undo) __hip_atomic_fetch_sub(p, one, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
-                    else __hip_atomic_fetch_add(p, one, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
-                }
-            }
-        };
-        constexpr int kBatch = NT * kUnroll;
-        if constexpr (MINW <= 4) {
-            // two register sets: the reads of one batch are in flight while the other is counted
-            u32x4 r_a[kUnroll], r_b[kUnroll];
-            uint32_t m_a[kUnroll], m_b[kUnroll];
-            if (total > 0) fetch(0, r_a, m_a);
-            for (int g0 = 0; g0 < total; g0 += 2 * kBatch) {
-                if (g0 + kBatch < total) fetch(g0 + kBatch, r_b, m_b);
-                process(r_a, m_a);
-                if (g0 + kBatch < total) {
-                    if (g0 + 2 * kBatch < total) fetch(g0 + 2 * kBatch, r_a, m_a);
-                    process(r_b, m_b);
-                }
-            }
-        } else {
-            // tight register budgets: one set; the other workgroups of the CU cover the reads
-            u32x4 r_a[kUnroll];
-            uint32_t m_a[kUnroll];
-            for (int g0 = 0; g0 < total; g0 += kBatch) {
-                fetch(g0, r_a, m_a);
-                process(r_a, m_a);
-            }
-        }
-        long long mine = 0;             // (summed per wavefront: the same total on every thread)
-        for (int s = lane; s < S; s += kWave) mine += (long long)max(0, s_rb[s] - s_ra[s]);
-        for (int o = kWave / 2; o > 0; o >>= 1) mine += __shfl_xor(mine, o, kWave);
-        return (unsigned long long)mine;
-    };
+    // index entries the scans looked at (same on every thread)
+    const unsigned long long scan_entries = (unsigned long long)n * (unsigned long long)I;
 
-    unsigned long long streamed = 0;     // entries streamed so far (same on every thread)
+    unsigned long long scanned = 0;      // entries scanned so far (same on every thread)
     bool shrunk = false;        // the previous epoch was undone
     bool undone_once = false;   // some epoch of this item was undone
     int epoch = 0;
     for (; epoch < kMaxEpochs; epoch++) {
+        fresh_thread_ids();
         // ---- 1. priority bound per composite ------------------------------------
         if (tid < a.M) { s_rho[tid] = kInfBits; s_K[tid] = 0; s_active[tid] = 0; s_hsum[tid] = 0.0f; }
         __syncthreads();
@@ -493,10 +402,10 @@ __global__ __launch_bounds__(NT, MINW) void traverse_block_kernel(QueryArgs a, B
                 s_rho[tid] = max(s_rho[tid], __builtin_bit_cast(uint32_t, hm));
         }
         __syncthreads();
-        phase(1);
+        phase(1); if (a.dense_cap < 0 && -a.dense_cap == 1 + 1) return; fresh_thread_ids();
         // ---- 2. how far each stream goes: all windows with priority <= bound ----
         {   // one group of lanes per stream; search window by window (twice the stride,
-            // then four times as much, ...) so that probes stay near what will be streamed
+            // then four times as much, ...) so that probes stay near where the epoch will end
             const int lg = min(3, floor_log2(kWave / ((S + kWaves - 1) / kWaves))), G = 1 << lg;
             const int slot = lane >> lg, sidx = wave * (kWave >> lg) + slot, g = lane - slot * G;
             const bool active = sidx < S;
@@ -528,17 +437,16 @@ __global__ __launch_bounds__(NT, MINW) void traverse_block_kernel(QueryArgs a, B
         bool all_done = true;
         for (int m = 0; m < a.M; m++) all_done = all_done && s_active[m] == 0;
         if (all_done) break;      // every stream was already exhausted before this epoch
-        phase(2);
+        phase(2); if (a.dense_cap < 0 && -a.dense_cap == 2 + 1) return; fresh_thread_ids();
 
-        // ---- 3. stream the new ranges ---------------------------------------------
-        streamed += stream_epoch(false);
+        // ---- 3. the points whose L windows are now all consumed ---------------------
+        scan_epoch();
+        scanned += scan_entries;
         __syncthreads();
-        collect_promotions();
-        __syncthreads();
-        phase(3);
+        phase(3); if (a.dense_cap < 0 && -a.dense_cap == 3 + 1) return; fresh_thread_ids();
         const uint32_t np = misc[kPromoCount];
         // too many promotions at once (or no room left beside the ones still waiting
-        // for the other composites): take the epoch back and retry with half the stride
+        // for the other composites): drop the epoch and retry with half the stride
         if (np > (uint32_t)y.promo_max || misc[kEventCount] + np > (uint32_t)y.event_cap) {
             bool minimal = true;
             for (int s2 = 0; s2 < S; s2++) minimal = minimal && s_stride[s2] <= 1;
@@ -549,15 +457,13 @@ __global__ __launch_bounds__(NT, MINW) void traverse_block_kernel(QueryArgs a, B
                 __syncthreads();
                 break;
             } else {
-                streamed += stream_epoch(true);
-                __syncthreads();
                 if (tid < S) s_c[tid] = s_cprev[tid];
                 if (tid < S) s_stride[tid] = max(1, s_stride[tid] / 2);
                 if (tid == 0) misc[kPromoCount] = 0;
                 shrunk = true;
                 undone_once = true;
                 __syncthreads();
-                phase(4);
+                phase(4); if (a.dense_cap < 0 && -a.dense_cap == 4 + 1) return; fresh_thread_ids();
                 continue;
             }
         }
@@ -685,7 +591,7 @@ __global__ __launch_bounds__(NT, MINW) void traverse_block_kernel(QueryArgs a, B
             }
         }
         __syncthreads();
-        phase(5);
+        phase(5); if (a.dense_cap < 0 && -a.dense_cap == 5 + 1) return; fresh_thread_ids();
         if (misc[kFail]) break;
 
         // ---- 5. replay promotions in (step, composite) order ----------------------
@@ -831,7 +737,7 @@ __global__ __launch_bounds__(NT, MINW) void traverse_block_kernel(QueryArgs a, B
             misc[kPromoCount] = 0;
         }
         __syncthreads();
-        phase(6);
+        phase(6); if (a.dense_cap < 0 && -a.dense_cap == 6 + 1) return; fresh_thread_ids();
 
         // ---- 6. distances of the accepted candidates, merged into the top-k ---------
         const int nacc = (int)misc[kAccCount];
@@ -870,7 +776,7 @@ __global__ __launch_bounds__(NT, MINW) void traverse_block_kernel(QueryArgs a, B
             if (tid == 0) misc[kAccCount] = 0;
             __syncthreads();
         }
-        phase(7);
+        phase(7); if (a.dense_cap < 0 && -a.dense_cap == 7 + 1) return; fresh_thread_ids();
         if (stop) break;
         if (may_hand_over && misc[kNumCand] + misc[kEventCount] >= (uint32_t)hand_over_at) {
             // (the stop hints still learn from it: the dense kernel records its stops too)
@@ -949,7 +855,7 @@ __global__ __launch_bounds__(NT, MINW) void traverse_block_kernel(QueryArgs a, B
     if (a.counters) {
         for (int o = 32; o > 0; o >>= 1) probes += (uint32_t)__shfl_xor((int)probes, o, kWave);
         if (lane == 0) atomicAdd(&misc[kProbes], probes);
-        if (tid == 0) { misc[kStreamedLo] = (uint32_t)streamed; misc[kStreamedHi] = (uint32_t)(streamed >> 32); }
+        if (tid == 0) { misc[kScannedLo] = (uint32_t)scanned; misc[kScannedHi] = (uint32_t)(scanned >> 32); }
         __syncthreads();
         if (tid == 0) {
             unsigned long long steps;   // outer steps the loop would have run (:458, :598-609)
@@ -966,7 +872,7 @@ __global__ __launch_bounds__(NT, MINW) void traverse_block_kernel(QueryArgs a, B
             } else {
                 steps = min(bound, maxw + 1);
             }
-            const unsigned long long st = ((unsigned long long)misc[kStreamedHi] << 32) | misc[kStreamedLo];
+            const unsigned long long st = ((unsigned long long)misc[kScannedHi] << 32) | misc[kScannedLo];
             atomicAdd(&a.counters[(int64_t)qi * 4 + 0], st);
             atomicAdd(&a.counters[(int64_t)qi * 4 + 1], (unsigned long long)misc[kNumCand]);
             atomicAdd(&a.counters[(int64_t)qi * 4 + 2], (unsigned long long)misc[kProbes]);
@@ -983,9 +889,8 @@ bool block_traversal_supported(const QueryArgs& a, size_t* lds_bytes) {
     const BlockLayout y = make_block_layout(a);
     if (lds_bytes) *lds_bytes = y.lds_bytes;
     const int I = a.M * a.L;
-    if (!a.inv || !a.lids || a.ppb > 65536) return false;
-    if (a.L > 255) return false;            // 4- and 8-bit visit counters only
-    if (4 * I > kBlockThreads || a.M > 64) return false;   // one thread per partial chunk of a stream
+    if (!a.inv || a.ppb > 65536) return false;             // positions inside a slice are 16-bit values
+    if (4 * I > kBlockThreads || a.M > 64) return false;   // lane groups per stream in the searches; composite number in 6 bits
     if (a.kcap > 512) return false;
     if (a.ppb >= (1 << 25)) return false;
     if ((int64_t)a.L * (a.ppb + 2 * (int64_t)a.T) >= 0x7fffffffLL) return false;   // steps fit 32 bits
@@ -1005,20 +910,23 @@ int query_block(const QueryArgs& a_in, hipStream_t s) {
         a.q_first = q0;
         a.q_count = min(per_launch, a_in.nq - q0);
         const int64_t items = block_items(a.xcds, a.B, a.q_count);
-#define DCIH_LAUNCH(CB, MW)                                                                        \
+#define DCIH_LAUNCH(MW)                                                                            \
     do {                                                                                           \
         static DeviceOnce once;                                                                    \
         const int rc_attr = once.run([]() -> int {                                                 \
-            DCIH_HIP(hipFuncSetAttribute((const void*)traverse_block_kernel<kBlockThreads, CB, MW>, \
+            DCIH_HIP(hipFuncSetAttribute((const void*)traverse_block_kernel<kBlockThreads, MW>,    \
                                          hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024)); \
             return 0;                                                                              \
         });                                                                                        \
         if (rc_attr) return rc_attr;                                                               \
-        hipLaunchKernelGGL((traverse_block_kernel<kBlockThreads, CB, MW>), dim3((unsigned)items),  \
+        hipLaunchKernelGGL((traverse_block_kernel<kBlockThreads, MW>), dim3((unsigned)items),      \
                            dim3(kBlockThreads), y.lds_bytes, s, a, y);                             \
     } while (0)
-        if (y.cbits == 4) { if (fit >= 6) DCIH_LAUNCH(4, 6); else if (fit >= 5) DCIH_LAUNCH(4, 5); else if (fit == 4) DCIH_LAUNCH(4, 4); else DCIH_LAUNCH(4, 3); }
-        else              { if (fit >= 6) DCIH_LAUNCH(8, 6); else if (fit >= 5) DCIH_LAUNCH(8, 5); else if (fit == 4) DCIH_LAUNCH(8, 4); else DCIH_LAUNCH(8, 3); }
+        // (measured on 1M x 128, 17858-point partitions: 5 -> 223 k, 6 -> 235 k, 7 and 8 -> 241 k queries/s)
+        int minw = fit >= 7 ? 7 : (fit < 3 ? 3 : fit);
+        if (const char* e = getenv("DCIH_BLOCK_MINW")) minw = atoi(e);
+        if (minw >= 8) DCIH_LAUNCH(8); else if (minw == 7) DCIH_LAUNCH(7); else if (minw == 6) DCIH_LAUNCH(6);
+        else if (minw == 5) DCIH_LAUNCH(5); else if (minw == 4) DCIH_LAUNCH(4); else DCIH_LAUNCH(3);
 #undef DCIH_LAUNCH
         DCIH_HIP(hipGetLastError());
     }

@@ -77,8 +77,14 @@ def test_merge_refuses_long_partitions(gpu):
     _capi.check(d._lib.dcih_set_option(d._dci_inst, _capi.OPT_APPEND, _capi.APPEND_MERGE))
     x = torch.randn(20000, 8, device="cuda")
     d.append(x)                                        # the first append has nothing to merge with
-    with pytest.raises(_capi.DCIError):
-        d.append(x)                                    # one partition of 40000 points
+    torch.cuda.synchronize()
+    free_before = torch.cuda.mem_get_info()[0]
+    for _ in range(3):
+        with pytest.raises(_capi.DCIError):
+            d.append(x)                                # one partition of 40000 points
+    torch.cuda.synchronize()
+    # a refused append allocates nothing it keeps (the buffers for 40000 rows would be 1.9 MB a call)
+    assert torch.cuda.mem_get_info()[0] >= free_before - (1 << 20)
     assert d.num_points == 20000
     _capi.check(d._lib.dcih_set_option(d._dci_inst, _capi.OPT_APPEND, _capi.APPEND_AUTO))
     d.append(x)                                        # left to choose, it sorts

@@ -21,6 +21,7 @@ import numpy as np
 import pytest
 import torch
 
+import bench
 from util import batch_fits, dense_fits, engine_index, engine_project, set_agreement
 
 pytestmark = pytest.mark.gpu
@@ -28,9 +29,8 @@ pytestmark = pytest.mark.gpu
 DIST_RTOL = 1e-5
 
 # the settings bench.py runs these configurations at (block_size, thread_size, outer)
-C3_SETTING = (400, 128, 100)
-C4_SETTING = (100, 64, 126)
-C5_SETTING = (900, 128, 10)
+C3_SETTING, C4_SETTING, C5_SETTING = ((bench.TUNED[c]["bs"], bench.TUNED[c]["ts"], bench.TUNED[c]["outer"])
+                                      for c in ("c3", "c4", "c5"))
 
 
 def _say(*a):
@@ -181,6 +181,25 @@ def test_c5_reduced_appends_against_oracle(gpu, oracle, batch_rows, B, T, outer)
     dci.free()
 
 
+def test_c5_reduced_at_the_full_size_operating_point(gpu, oracle):
+    """The regime the benchmark runs C5 in at 20M points: 22223 points per partition, windows of
+    128, 10 outer iterations, L = 15, k = 50 (the stop is set by c0 >= 50: thousands of promotions
+    per partition).  Three such partitions against the oracle."""
+    from dciknn_cuda_amd import workloads
+    B20, T, outer = C5_SETTING
+    ppb = -(-20_000_000 // B20)
+    M, L, k, dim, nq, B = 2, 15, 50, 64, 24, 3
+    n = B * ppb
+    Q = workloads.c5_queries(nq=nq).numpy()
+    X = workloads.c5_batch(0, n=n).numpy()
+    dci = gpu.DCI(dim, M, L, B, T, seed=56)
+    dci.add(torch.from_numpy(X).cuda())
+    assert -(-n // B) == ppb
+    _l1(gpu, oracle, dci, X, Q, M, L, B, T, k, outer, ["step", "batch", "dense", "auto"])
+    _l2(oracle, dci, X, Q, M, L, B, T, k, outer)
+    dci.free()
+
+
 # ------------------------------------------------------------------ full size, properties
 def test_c3_full_size(gpu):
     from dciknn_cuda_amd import workloads
@@ -241,6 +260,7 @@ def test_c5_full_size_appends_equal_one_add(gpu):
     _say("c5 full: 20 appends (with generation) in %.1f s" % (time.time() - t))
     recalls.append(_properties(grown, Xd, Qd, k, outer, 0.9))
     _say("c5 full: recall@50 after 1, 10, 20 batches", recalls)
+    _kernels_agree(grown, Qd[:6].contiguous(), k, outer, ["step", "dense", "auto"])
     one = gpu.DCI(dim, 2, 15, B, T, directions=grown.directions)
     one.add(Xd)
     for mode in ("auto", "step"):

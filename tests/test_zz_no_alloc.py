@@ -1,7 +1,8 @@
 """dcih_query_noalloc (all scratch from the library's fixed device array, no
 allocation) against dcih_query on the same index and queries: identical ids,
 distances and counters, on two calls in a row, the second with a smaller input,
-plus its size limit."""
+plus its size limit, and the one kind of shape where the two agree as sets and to
+1e-5 in the distances instead of bit for bit."""
 import numpy as np
 import pytest
 import torch
@@ -46,6 +47,26 @@ def test_noalloc_equals_query_twice_second_smaller(gpu, traversal):
         want = _call(dci, lib.dcih_query, Q, k, outer, B, T, blind=1)
         got = _call(dci, lib.dcih_query_noalloc, Q, k, outer, B, T, blind=1)
         assert torch.equal(got[0], want[0]) and torch.equal(got[1], want[1])
+    dci.free()
+
+
+def test_noalloc_on_a_shape_that_runs_dry(gpu):
+    """The reference's example configuration (3000 points in 100 partitions, 5000 iterations):
+    the stop rule cannot fire, dcih_query ranks all points directly, dcih_query_noalloc runs the
+    traversal.  Same neighbours; the distances are summed in another order and agree to 1e-5."""
+    from dciknn_cuda_amd import workloads
+    X, Q = workloads.c1()
+    dim, M, L, B, T, k, outer = 100, 2, 10, 100, 10, 10, 5000
+    dci = gpu.DCI(dim, M, L, B, T, seed=4)
+    dci.add(X.cuda())
+    for Qd in (Q.cuda(), Q[:77].contiguous().cuda()):
+        want = _call(dci, dci._lib.dcih_query, Qd, k, outer, B, T)
+        got = _call(dci, dci._lib.dcih_query_noalloc, Qd, k, outer, B, T)
+        assert torch.allclose(got[1], want[1], rtol=1e-5, atol=0.0)
+        a, b = got[0].cpu().numpy(), want[0].cpu().numpy()
+        agree = np.mean([len(set(x.tolist()) & set(y.tolist())) / k for x, y in zip(a, b)])
+        assert agree >= 0.999, agree
+        assert torch.equal(got[2][:, 1], want[2][:, 1]) and torch.equal(got[2][:, 3], want[2][:, 3])
     dci.free()
 
 
