@@ -8,7 +8,6 @@
 // several per query.
 #include <algorithm>
 #include <cmath>
-#include <cstdlib>
 #include <cstring>
 #include <new>
 #include <string>
@@ -640,7 +639,6 @@ static int query_impl(dcih_index* h, int dim, int num_queries, const float* d_qu
     a.dense_count = a.redo_count + 1;         // one length per die, cleared together with redo_count
     a.dense_items = dense_lists ? (int32_t*)(base + qp_bytes + part_bytes + gs_bytes + redo_bytes + 256) : nullptr;
 
-    if (const char* e = getenv("DCIH_STOP_PHASE")) { if (!a.dense_items) a.dense_cap = -(int64_t)(atoi(e) + 1); }   // TEMP
     mark(h, DCIH_T_QPROJECT, 0, s);
     rc = project(h->d_dirs, I, d_query, num_queries, dim, d_qproj, num_queries, s);
     mark(h, DCIH_T_QPROJECT, 1, s);

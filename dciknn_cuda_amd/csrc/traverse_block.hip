@@ -33,8 +33,6 @@
 // many points at once is dropped and retried smaller.  Whatever does not fit the
 // fixed LDS tables is handed to the step-by-step kernel through a redo list, so
 // results never depend on which kernel produced them.
-#include <stdlib.h>
-
 #include <type_traits>
 
 #include "common.h"
@@ -47,9 +45,10 @@ namespace {
 
 constexpr int kMaxEpochs = 100000;
 
+
 enum Misc {   // 32-bit scalars shared by the workgroup
     kPromoCount = 0, kEventCount, kAccCount, kFail, kStop, kC0, kStopStepLo, kStopStepHi,
-    kArmedLo, kArmedHi, kScannedLo, kScannedHi, kArmed, kNumCand, kTopN, kProbes, kMiscWords
+    kArmedLo, kArmedHi, kScannedLo, kScannedHi, kArmed, kNumCand, kTopN, kProbes, kHintSteps, kHintPromos, kMiscWords
 };
 
 struct BlockLayout {
@@ -145,6 +144,18 @@ __global__ __launch_bounds__(NT, MINW) void traverse_block_kernel(QueryArgs a, B
         lane = tid & (kWave - 1);
         wave = tid / kWave;
     };
+    // For the same reason every phase ends in an exit that is never taken but that the compiler
+    // cannot rule out (PHASE_END): loads and address arithmetic of the phases after it are then
+    // not moved up across it, or out of the epoch loop.  Without the two, the five-workgroup
+    // variant keeps 244 bytes per lane in scratch instead of 12 and the kernel runs a quarter slower.
+#define PHASE_END(which)                                 \
+    do {                                                 \
+        phase(which);                                    \
+        int leave_now = 0;                               \
+        asm volatile("" : "+s"(leave_now));              \
+        if (leave_now) return;                           \
+        fresh_thread_ids();                              \
+    } while (0)
     constexpr int kWaves = NT / kWave;
     // optional phase profile: thread 0 adds the 100 MHz ticks each phase took
     unsigned long long tick = a.phase_ticks ? wall_clock64() : 0ull;
@@ -187,7 +198,20 @@ __global__ __launch_bounds__(NT, MINW) void traverse_block_kernel(QueryArgs a, B
             a.dense_items[(int64_t)x * a.dense_cap + sl] = (int32_t)item;
         }
     };
-    if (may_hand_over && a.stop_hint && a.stop_hint[a.B + b] >= (float)hand_over_at) {
+    // usual stop step and promotions at the stop: read by one thread, because other workgroups
+    // are updating them and every thread must decide alike
+    if (threadIdx.x < kMiscWords) misc[threadIdx.x] = 0;
+    __syncthreads();
+    if (threadIdx.x == 0 && a.stop_hint) {
+        float steps, promotions;
+        usual_stop(a.stop_hint, a.B, b, steps, promotions);
+        misc[kHintSteps] = __builtin_bit_cast(uint32_t, steps);
+        misc[kHintPromos] = __builtin_bit_cast(uint32_t, promotions);
+    }
+    __syncthreads();
+    const float hint = __builtin_bit_cast(float, misc[kHintSteps]);
+    const float hint_promos = __builtin_bit_cast(float, misc[kHintPromos]);
+    if (may_hand_over && hint_promos >= (float)hand_over_at) {
         hand_to_dense();
         return;
     }
@@ -200,7 +224,6 @@ __global__ __launch_bounds__(NT, MINW) void traverse_block_kernel(QueryArgs a, B
     // ---- set-up ---------------------------------------------------------------
     for (int w = tid; w < y.flag_words; w += NT) seen[w] = 0;
     for (int j = tid; j < a.dim; j += NT) s_q[j] = a.query[(int64_t)qi * a.dim + j];
-    if (tid < kMiscWords) misc[tid] = 0;
     uint32_t probes = 0;
     {   // positioning search (:279-297): first position whose key is not below qp,
         // one group of lanes per simple index
@@ -228,8 +251,8 @@ __global__ __launch_bounds__(NT, MINW) void traverse_block_kernel(QueryArgs a, B
     // (its local density), scaled so that every composite lands on the same step
     // count: a composite left behind would keep the promotions of the others
     // waiting.  The total doubles from epoch to epoch until one has to be undone.
-    // hint = running average of the step at which earlier queries stopped in this
-    // partition; it only steers epoch sizes, never results.  The first jump aims
+    // hint = average step at which earlier queries stopped in this partition (record_stop);
+    // it only steers epoch sizes, never results.  The first jump aims
     // 12 % past it.  The number of points whose counters are complete grows like a
     // high power (L) of the steps taken, so stop steps of one partition scatter
     // little and most items finish in one epoch (12 % more steps bring about three
@@ -242,8 +265,6 @@ __global__ __launch_bounds__(NT, MINW) void traverse_block_kernel(QueryArgs a, B
     constexpr float kHintGrow = 1.06f;
     const float kPromoAim = 0.6f * (float)y.promo_max;
     const float inv_L = 1.0f / (float)a.L;
-    const float hint = a.stop_hint ? a.stop_hint[b] : 0.0f;
-    const float hint_promos = a.stop_hint ? a.stop_hint[a.B + b] : 0.0f;
     const float kHintFirst = fminf(1.12f,
         fast_pow(kPromoAim / fmaxf(1.0f, hint_promos > 0.0f ? hint_promos : (float)a.k_stop * (float)T), inv_L));
     {
@@ -255,7 +276,7 @@ __global__ __launch_bounds__(NT, MINW) void traverse_block_kernel(QueryArgs a, B
         if (tid < a.M) s_Kprev[tid] = 0;
     }
     __syncthreads();
-    phase(0); if (a.dense_cap < 0 && -a.dense_cap == 0 + 1) return; fresh_thread_ids();
+    PHASE_END(0);
 
     auto load_stream = [&](int s) {
         Stream st;
@@ -402,7 +423,7 @@ __global__ __launch_bounds__(NT, MINW) void traverse_block_kernel(QueryArgs a, B
                 s_rho[tid] = max(s_rho[tid], __builtin_bit_cast(uint32_t, hm));
         }
         __syncthreads();
-        phase(1); if (a.dense_cap < 0 && -a.dense_cap == 1 + 1) return; fresh_thread_ids();
+        PHASE_END(1);
         // ---- 2. how far each stream goes: all windows with priority <= bound ----
         {   // one group of lanes per stream; search window by window (twice the stride,
             // then four times as much, ...) so that probes stay near where the epoch will end
@@ -437,13 +458,13 @@ __global__ __launch_bounds__(NT, MINW) void traverse_block_kernel(QueryArgs a, B
         bool all_done = true;
         for (int m = 0; m < a.M; m++) all_done = all_done && s_active[m] == 0;
         if (all_done) break;      // every stream was already exhausted before this epoch
-        phase(2); if (a.dense_cap < 0 && -a.dense_cap == 2 + 1) return; fresh_thread_ids();
+        PHASE_END(2);
 
         // ---- 3. the points whose L windows are now all consumed ---------------------
         scan_epoch();
         scanned += scan_entries;
         __syncthreads();
-        phase(3); if (a.dense_cap < 0 && -a.dense_cap == 3 + 1) return; fresh_thread_ids();
+        PHASE_END(3);
         const uint32_t np = misc[kPromoCount];
         // too many promotions at once (or no room left beside the ones still waiting
         // for the other composites): drop the epoch and retry with half the stride
@@ -463,7 +484,7 @@ __global__ __launch_bounds__(NT, MINW) void traverse_block_kernel(QueryArgs a, B
                 shrunk = true;
                 undone_once = true;
                 __syncthreads();
-                phase(4); if (a.dense_cap < 0 && -a.dense_cap == 4 + 1) return; fresh_thread_ids();
+                PHASE_END(4);
                 continue;
             }
         }
@@ -591,7 +612,7 @@ __global__ __launch_bounds__(NT, MINW) void traverse_block_kernel(QueryArgs a, B
             }
         }
         __syncthreads();
-        phase(5); if (a.dense_cap < 0 && -a.dense_cap == 5 + 1) return; fresh_thread_ids();
+        PHASE_END(5);
         if (misc[kFail]) break;
 
         // ---- 5. replay promotions in (step, composite) order ----------------------
@@ -737,7 +758,7 @@ __global__ __launch_bounds__(NT, MINW) void traverse_block_kernel(QueryArgs a, B
             misc[kPromoCount] = 0;
         }
         __syncthreads();
-        phase(6); if (a.dense_cap < 0 && -a.dense_cap == 6 + 1) return; fresh_thread_ids();
+        PHASE_END(6);
 
         // ---- 6. distances of the accepted candidates, merged into the top-k ---------
         const int nacc = (int)misc[kAccCount];
@@ -776,7 +797,7 @@ __global__ __launch_bounds__(NT, MINW) void traverse_block_kernel(QueryArgs a, B
             if (tid == 0) misc[kAccCount] = 0;
             __syncthreads();
         }
-        phase(7); if (a.dense_cap < 0 && -a.dense_cap == 7 + 1) return; fresh_thread_ids();
+        PHASE_END(7);
         if (stop) break;
         if (may_hand_over && misc[kNumCand] + misc[kEventCount] >= (uint32_t)hand_over_at) {
             // (the stop hints still learn from it: the dense kernel records its stops too)
@@ -838,17 +859,9 @@ __global__ __launch_bounds__(NT, MINW) void traverse_block_kernel(QueryArgs a, B
         atomicAdd(&a.phase_ticks[8], (unsigned long long)epoch + 1);
         atomicAdd(&a.phase_ticks[9], 1ull);
     }
-    if (a.stop_hint && tid == 0 && misc[kStop]) {
-        const float cur = (float)((((unsigned long long)misc[kStopStepHi] << 32) | misc[kStopStepLo]) + 1);
-        // racy on purpose: any recent value will do.  The mean of the first 50 stops, then an
-        // exponential average with weight 1/50 (a smooth hint wastes the fewest epochs).
-        const float seen_stops = a.stop_hint[2 * a.B + b];
-        const float w = 1.0f / fminf(seen_stops + 1.0f, 50.0f);
-        a.stop_hint[2 * a.B + b] = fminf(seen_stops + 1.0f, 1.0e6f);
-        a.stop_hint[b] += w * (cur - a.stop_hint[b]);
-        const float curp = (float)(misc[kNumCand] + misc[kEventCount]);
-        a.stop_hint[a.B + b] += w * (curp - a.stop_hint[a.B + b]);
-    }
+    if (a.stop_hint && tid == 0 && misc[kStop])
+        record_stop(a.stop_hint, a.B, b, (float)((((unsigned long long)misc[kStopStepHi] << 32) | misc[kStopStepLo]) + 1),
+                    (float)(misc[kNumCand] + misc[kEventCount]));
     // ---- results -------------------------------------------------------------------
     const int topn = (int)misc[kTopN];
     for (int j = tid; j < a.kcap; j += NT) part_out[j] = j < topn ? sortbuf[j] : ~0ull;
@@ -882,6 +895,8 @@ __global__ __launch_bounds__(NT, MINW) void traverse_block_kernel(QueryArgs a, B
 }
 
 constexpr int kBlockThreads = 256;
+
+#undef PHASE_END
 
 }  // namespace
 
@@ -924,7 +939,6 @@ int query_block(const QueryArgs& a_in, hipStream_t s) {
     } while (0)
         // (measured on 1M x 128, 17858-point partitions: 5 -> 223 k, 6 -> 235 k, 7 and 8 -> 241 k queries/s)
         int minw = fit >= 7 ? 7 : (fit < 3 ? 3 : fit);
-        if (const char* e = getenv("DCIH_BLOCK_MINW")) minw = atoi(e);
         if (minw >= 8) DCIH_LAUNCH(8); else if (minw == 7) DCIH_LAUNCH(7); else if (minw == 6) DCIH_LAUNCH(6);
         else if (minw == 5) DCIH_LAUNCH(5); else if (minw == 4) DCIH_LAUNCH(4); else DCIH_LAUNCH(3);
 #undef DCIH_LAUNCH

@@ -96,6 +96,25 @@ __device__ inline int group_partition_point(int lo, int hi, bool active, int lg,
     }
     return lo;
 }
+// Where traversals of a partition usually stop: stop_hint is [3][B] -- the sum of the stop
+// steps, the sum of the promotions at the stop, and the number of stops recorded, per
+// partition.  Many workgroups record at once, so the sums are formed by atomic additions; a
+// partition stops recording after kHintStops stops, which makes the averages (and with them
+// the sizes of the batch kernel's epochs) the same from then on.  They steer work, never results.
+constexpr float kHintStops = 4096.0f;
+__device__ inline void record_stop(float* stop_hint, int B, int b, float steps, float promotions) {
+    if (stop_hint[2 * B + b] >= kHintStops) return;
+    atomicAdd(&stop_hint[b], steps);
+    atomicAdd(&stop_hint[B + b], promotions);
+    atomicAdd(&stop_hint[2 * B + b], 1.0f);
+}
+// (average stop step, average promotions at the stop); zeros while nothing is recorded.  The
+// three words are read at different moments, so the averages can be off by a stop's share.
+__device__ inline void usual_stop(const float* stop_hint, int B, int b, float& steps, float& promotions) {
+    const float stops = stop_hint[2 * B + b];
+    steps = stops > 0.0f ? stop_hint[b] / stops : 0.0f;
+    promotions = stops > 0.0f ? stop_hint[B + b] / stops : 0.0f;
+}
 // x^y for x > 0 from the hardware's log2 / exp2 approximations (epoch sizing only)
 __device__ inline float fast_pow(float x, float y) { return __builtin_amdgcn_exp2f(__builtin_amdgcn_logf(x) * y); }
 __host__ __device__ inline int floor_log2(int v) { int l = 0; while ((2 << l) <= v) l++; return l; }
