@@ -20,8 +20,8 @@ steps run on the final index.  Prints ONE JSON line:
   roofline       the kernel that took most of the step, against the limit that binds
                  it: `frac` is always achieved / peak of that limit (<= 1).  For the
                  batch traversal kernel the limit is vector-ALU issue (lane
-                 instructions), for the dense traversal kernel HBM bytes (candidate
-                 rows + index slices); the figure by the reference's 8-byte index
+                 instructions; its L2-side figure is given beside it), for the dense
+                 traversal kernel HBM bytes (candidate rows + index slices); the figure by the reference's 8-byte index
                  entries is kept as contract_bytes_* and is not a bound.  `traffic`
                  = HBM bytes per launch from profiles/hbm_traffic.json (rocprofv3
                  counter runs of this file), null when that file has no entry for
@@ -29,6 +29,9 @@ steps run on the final index.  Prints ONE JSON line:
   cpu_baseline   the CPU restatement of the reference algorithm on this box's host
                  cores on a bounded sample of the same workload
   first_call, outer_sweep, blind   extra measurements outside the timed steps
+  other_configs  (default run only) compact legs of the other workloads and of this one at
+                 the reference's constructor defaults, each from a run of this file in a
+                 process of its own: value, recall, setting, kernel times, roofline fraction
 """
 import argparse
 import json
@@ -42,9 +45,22 @@ sys.path.insert(0, ROOT)
 HBM_PEAK_GBS = 8000.0   # MI355X HBM3E
 # vector-ALU issue peak: 256 CUs x 4 SIMDs x 16 lanes x 2.4 GHz lane instructions per second
 VALU_PEAK_GOPS = 256 * 4 * 16 * 2.4
-# lane instructions the batch kernel cannot do without per streamed index entry: its share
-# of the 16-byte id read, the id's extraction, the counter's address, the LDS update
-MIN_INSTR_PER_ENTRY = 4.0
+# lane instructions the batch kernel cannot do without per index entry it scans: three packed
+# 16-bit instructions per PAIR of entries (position - run start, minus run length with
+# saturation, running maximum)
+MIN_INSTR_PER_ENTRY = 1.5
+# L2 -> CU read peak: 8 XCDs x 16 channels x 128 B per clock x 2.4 GHz
+L2_PEAK_GBS = 8 * 16 * 128 * 2.4
+# compact legs of the other workloads (and of this one at the reference's own defaults) that the
+# default run adds to its line: (name, extra arguments)
+OTHER_LEGS = [
+    ("c1", ["--config", "c1"]),
+    ("c2_reference_defaults_outer500", ["--config", "c2", "--bs", "100", "--ts", "10", "--outer", "500"]),
+    ("c2_reference_defaults_outer5000", ["--config", "c2", "--bs", "100", "--ts", "10", "--outer", "5000"]),
+    ("c4", ["--config", "c4"]),
+    ("c3", ["--config", "c3"]),
+    ("c5", ["--config", "c5"]),
+]
 
 # (block_size, thread_size, num_outer_iterations) used when none are given: the fastest
 # setting found that meets the workload's recall target (RECALL_TARGET; c5 has none and runs
@@ -85,6 +101,9 @@ def parse():
     p.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     p.add_argument("--no-extras", action="store_true",
                    help="skip first_call, outer_sweep and blind (profiling runs)")
+    p.add_argument("--no-others", action="store_true",
+                   help="skip the compact legs of the other workloads that the default run (c2 at its "
+                        "tuned setting, extras on) appends as other_configs")
     p.add_argument("--build-reps", type=int, default=3)
     p.add_argument("--traversal", default="auto", choices=["auto", "step", "batch", "dense"])
     p.add_argument("--c5-batches", type=int, default=20, help="batches of the incremental workload")
@@ -248,7 +267,7 @@ def main():
     # ---- first call of this query shape: nothing learnt about where traversals stop ----
     first_call = None
     if not a.no_extras:
-        dci.query(Qd, k, outer)                  # workspace and kernel attributes in place
+        dci.query(Qd, k, outer, return_int=True)                  # workspace and kernel attributes in place
         _capi.check(lib.dcih_set_option(dci._dci_inst, _capi.OPT_FORGET_HINTS, 0))
         torch.cuda.synchronize()
         t0 = time.perf_counter()
@@ -262,7 +281,7 @@ def main():
 
     # ---- query: warmup, then K timed steps ----------------------------------------
     for _ in range(a.warmup):
-        dci.query(Qd, k, outer)
+        dci.query(Qd, k, outer, return_int=True)
     tsum = np.zeros(_capi.NUM_TIMERS)
     torch.cuda.synchronize()
     t0 = time.perf_counter()
@@ -329,8 +348,16 @@ def main():
     if kernel == "traverse_block_kernel":
         roofline = dict(bound="valu", kernel=kernel, achieved=valu_gops, peak=VALU_PEAK_GOPS,
                         unit="G lane-instr/s", frac=valu_gops / VALU_PEAK_GOPS,
-                        model="%.0f lane instructions per index entry streamed x %.4g entries per launch"
-                              % (MIN_INSTR_PER_ENTRY, float(own[0]) * nq))
+                        model="%.1f lane instructions per index entry scanned (3 packed 16-bit instructions per "
+                              "pair) x %.4g entries per launch" % (MIN_INSTR_PER_ENTRY, float(own[0]) * nq))
+        # memory side of the same kernel: what it reads through L2 in this layout -- 2 bytes per
+        # entry scanned (16-bit position), 4 per key read, the candidates' rows
+        l2_bytes = nq * (2.0 * float(own[0]) + 4.0 * float(own[2]) + 4.0 * dim * C)
+        roofline.update(l2_model_bytes_per_launch=l2_bytes,
+                        l2_model_gbs=l2_bytes / (launch_ms * 1e-3) / 1e9,
+                        l2_frac=l2_bytes / (launch_ms * 1e-3) / 1e9 / L2_PEAK_GBS,
+                        l2_model="2 B per index entry scanned + 4 B per key read + candidate rows, against "
+                                 "%.0f GB/s (8 XCDs x 16 channels x 128 B/clk x 2.4 GHz)" % L2_PEAK_GBS)
     else:
         roofline = dict(bound="hbm", kernel=kernel, achieved=hbm_gbs, peak=HBM_PEAK_GBS,
                         unit="GB/s", frac=hbm_gbs / HBM_PEAK_GBS,
@@ -373,7 +400,7 @@ def main():
             outer_sweep = []
             say("sweep of num_outer_iterations")
             for o in (500, 1000, 2000, 5000, 10000, 20000):
-                dci.query(Qd, k, o)
+                dci.query(Qd, k, o, return_int=True)
                 torch.cuda.synchronize()
                 t0 = time.perf_counter()
                 for _ in range(2):
@@ -382,7 +409,7 @@ def main():
                 dt = (time.perf_counter() - t0) / 2
                 outer_sweep.append(dict(num_outer_iterations=o, queries_per_s=nq / dt,
                                         recall_at_k=workloads.recall_at_k(oi[:nrec], truth)))
-            dci.query(Qd, k, outer)
+            dci.query(Qd, k, outer, return_int=True)
         if min(10 * k, outer) <= 8192:
             # no distances: per query the first min(10k, outer) promoted candidates by promoting step
             nqb = min(nq, legs["blind"])
@@ -445,6 +472,38 @@ def main():
                    exact_cdist_topk_queries_per_s=nex / t_exact * scale,
                    host_cpus=os.cpu_count(), torch_threads=torch.get_num_threads())
 
+    # ---- the other workloads, compactly (default run only) -----------------------------
+    others = None
+    default_run = (config == "c2" and not a.no_extras and not a.no_others and a.traversal == "auto"
+                   and all(getattr(a, key) is None for key in ("bs", "ts", "outer", "nq", "n")))
+    if default_run:
+        import subprocess
+        dci.free()
+        del Xd, Qd
+        torch.cuda.empty_cache()
+        others = {}
+        for name, extra in OTHER_LEGS:
+            say("other configuration:", name)
+            t0 = time.perf_counter()
+            try:
+                r = subprocess.run([sys.executable, os.path.abspath(__file__), "--steps", "2", "--warmup", "1",
+                                    "--no-cpu", "--no-extras", "--build-reps", "1"] + extra,
+                                   capture_output=True, text=True, timeout=280)
+                if r.returncode != 0 or not r.stdout.strip():
+                    raise RuntimeError("exit code %d: %s" % (r.returncode, r.stderr.strip()[-300:]))
+                line = json.loads(r.stdout.strip().splitlines()[-1])
+                others[name] = dict(
+                    value=line["value"], unit=line["unit"], workload=line["config"]["workload"],
+                    block_size=line["config"]["block_size"], thread_size=line["config"]["thread_size"],
+                    num_outer_iterations=line["config"]["num_outer_iterations"],
+                    recall_at_k=line["recall_at_k"], recall_target=line["recall_target"],
+                    ms_per_step=line["ms_per_step"], kernel_ms=line["kernel_ms"],
+                    build_points_per_s=line["build_points_per_s"],
+                    roofline={key: line["roofline"][key] for key in ("bound", "kernel", "frac", "achieved", "peak", "unit")},
+                    seconds=time.perf_counter() - t0)
+            except Exception as exc:       # a leg that fails or runs out of time is reported as such
+                others[name] = dict(error="%s: %s" % (type(exc).__name__, str(exc)[:200]))
+
     out = {
         "metric": "queries/sec at recall@10>=0.95, 1Mx128 fp32 k=10; index build points/sec"
                   if config == "c2" else "queries/sec; index build points/sec",
@@ -468,6 +527,7 @@ def main():
         "outer_sweep": outer_sweep,
         "blind": blind,
         "per_size": per_size,
+        "other_configs": others,
         "roofline": roofline,
         "cpu_baseline": cpu,
     }

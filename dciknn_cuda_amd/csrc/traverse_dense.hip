@@ -145,9 +145,27 @@ __global__ __launch_bounds__(kDT, WPS) void traverse_dense_kernel(QueryArgs a, D
     uint16_t* s_wlist = reinterpret_cast<uint16_t*>(smem + y.off_wlist);   // per wavefront: kWlist candidates
     int* s_segw = s_segstream + 2 * a.L;                              // table place of a segment's window 0
 
-    const int tid = threadIdx.x;
-    const int lane = tid & (kWave - 1);
-    const int wave = tid / kWave;
+    // The thread numbers are made opaque again at the start of every phase, and every phase ends
+    // in an exit that is never taken but that the compiler cannot rule out (PHASE_END): otherwise
+    // each phase's lane groupings, per-thread addresses and loop-invariant loads are computed
+    // once, ahead of the loop over the items, and carried through every other phase in registers
+    // or scratch.
+    int tid = threadIdx.x;
+    int lane = tid & (kWave - 1);
+    int wave = tid / kWave;
+    auto fresh_thread_ids = [&]() {
+        asm volatile("" : "+v"(tid));
+        lane = tid & (kWave - 1);
+        wave = tid / kWave;
+    };
+#define PHASE_END(which)                                 \
+    do {                                                 \
+        phase(which);                                    \
+        int leave_now = 0;                               \
+        asm volatile("" : "+s"(leave_now));              \
+        if (leave_now) return;                           \
+        fresh_thread_ids();                              \
+    } while (0)
     const int I = a.M * a.L;
     const int T = a.T;
     const int X = a.xcds;
@@ -208,7 +226,7 @@ __global__ __launch_bounds__(kDT, WPS) void traverse_dense_kernel(QueryArgs a, D
             }
         }
         __syncthreads();
-        phase(0);
+        PHASE_END(0);
 
         unsigned long long maxw = 0;             // most windows any composite has
         for (int m = 0; m < a.M; m++) {
@@ -329,7 +347,7 @@ __global__ __launch_bounds__(kDT, WPS) void traverse_dense_kernel(QueryArgs a, D
                 if (lane == 0) { atomicOr(&misc[dOr], vor); atomicAnd(&misc[dAnd], vand); }
             }
             __syncthreads();
-            phase(1);
+            PHASE_END(1);
             // the step of every window: its place in the sorted order, stored doubled with bit 0
             // set: a lookup subtracts one where the point is not the window's first lane, which
             // leaves the lane-0 flag beside the step
@@ -376,7 +394,7 @@ __global__ __launch_bounds__(kDT, WPS) void traverse_dense_kernel(QueryArgs a, D
                 }
             }
             __syncthreads();
-            phase(2);
+            PHASE_END(2);
 
             // ---- every point: the latest of the steps of its L windows ------------------
             // A thread takes eight consecutive points at a time: their positions in one simple
@@ -538,7 +556,7 @@ __global__ __launch_bounds__(kDT, WPS) void traverse_dense_kernel(QueryArgs a, D
                 else run(std::integral_constant<int, 2>{});
             }
             __syncthreads();
-            phase(3);
+            PHASE_END(3);
         }
         if (misc[dFail]) {      // does not fit the tables: the step-by-step kernel takes the item
             if (tid == 0) {
@@ -596,7 +614,7 @@ __global__ __launch_bounds__(kDT, WPS) void traverse_dense_kernel(QueryArgs a, D
         }
         const uint32_t t_lim = (uint32_t)min(t_stop, (unsigned long long)0x7ffe);   // every real step is below 0x7fff
         __syncthreads();                                    // the histogram's room is free again
-        phase(4);
+        PHASE_END(4);
 
         // ---- distances of the candidates, k best ---------------------------------------
         // Every wavefront walks a quarter of the points; a candidate whose packed
@@ -788,7 +806,7 @@ __global__ __launch_bounds__(kDT, WPS) void traverse_dense_kernel(QueryArgs a, D
         }
         if (lane == 0) atomicAdd(&misc[dCand], ncand);
         for (int j = tid; j < a.kcap; j += kDT) part_out[j] = j < topn ? sortbuf[j] : ~0ull;
-        phase(5);
+        PHASE_END(5);
         if (a.phase_ticks && tid == 0) atomicAdd(&a.phase_ticks[9], 1ull);
 
         // ---- hints for the batch kernel's routing, counters -----------------------------
@@ -810,6 +828,8 @@ __global__ __launch_bounds__(kDT, WPS) void traverse_dense_kernel(QueryArgs a, D
         }
     }
 }
+
+#undef PHASE_END
 
 }  // namespace
 
