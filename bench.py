@@ -267,6 +267,7 @@ def main():
     # ---- first call of this query shape: nothing learnt about where traversals stop ----
     first_call = None
     if not a.no_extras:
+        say("first call of the query shape")
         dci.query(Qd, k, outer, return_int=True)                  # workspace and kernel attributes in place
         _capi.check(lib.dcih_set_option(dci._dci_inst, _capi.OPT_FORGET_HINTS, 0))
         torch.cuda.synchronize()
@@ -280,6 +281,7 @@ def main():
         _capi.check(lib.dcih_set_option(dci._dci_inst, _capi.OPT_FORGET_HINTS, 0))
 
     # ---- query: warmup, then K timed steps ----------------------------------------
+    say("warm-up and timed steps")
     for _ in range(a.warmup):
         dci.query(Qd, k, outer, return_int=True)
     tsum = np.zeros(_capi.NUM_TIMERS)
@@ -400,6 +402,7 @@ def main():
             outer_sweep = []
             say("sweep of num_outer_iterations")
             for o in (500, 1000, 2000, 5000, 10000, 20000):
+                say("  num_outer_iterations", o)
                 dci.query(Qd, k, o, return_int=True)
                 torch.cuda.synchronize()
                 t0 = time.perf_counter()

@@ -427,8 +427,14 @@ int query(const QueryArgs& a_in, hipStream_t s, hipEvent_t* ev, bool* ran) {
         // whatever those kernels handed back goes through the step-by-step kernel
         a.item_list = a.redo_items;
         a.item_count = a.redo_count;
-        const int64_t grid = min((int64_t)a.nq * a.B, (int64_t)1024);
-        hipLaunchKernelGGL(traverse_kernel<true>, dim3((unsigned)grid), dim3(kWave), y.lds_bytes, s, a, y);
+        if (y.lds_counters) {
+            const int64_t grid = min((int64_t)a.nq * a.B, (int64_t)1024);
+            hipLaunchKernelGGL(traverse_kernel<true>, dim3((unsigned)grid), dim3(kWave), y.lds_bytes, s, a, y);
+        } else {      // partitions whose visit counters do not fit LDS: a slice of global scratch per workgroup
+            if (!a.gscratch) return fail(-1, "query: counter scratch missing");
+            const int64_t grid = min(traverse_grid(a, y), (int64_t)1024);
+            hipLaunchKernelGGL(traverse_kernel<false>, dim3((unsigned)grid), dim3(kWave), y.lds_bytes, s, a, y);
+        }
     } else {
         const int64_t grid = traverse_grid(a, y);
         if (y.lds_counters) {

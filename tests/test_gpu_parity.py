@@ -187,6 +187,7 @@ CASES = [
     (40000, 16, 24, 2, 12, 4, 12, 10, 200, "normal"),       # 10032 windows per composite: the largest dense tables
     (3000, 8, 512, 2, 4, 3, 16, 10, 5, "normal"),           # long rows: two 1 KiB pieces
     (3000, 8, 1100, 2, 4, 3, 16, 10, 5, "normal"),          # long rows: five pieces, the last one short
+    (120000, 8, 16, 3, 16, 2, 8, 10, 30, "normal"),         # 60000-point partitions, 48 indices: the step kernel's counters leave LDS, the batch kernel's flags do not
 ]
 
 
