@@ -126,7 +126,6 @@ struct dcih_index {
     float* d_skeys = nullptr;           // [I][n]
     int32_t* d_sids = nullptr;          // [I][n]
     uint16_t* d_inv = nullptr;          // [I][n] position of each point in its sorted slice (partitions <= 65536 points)
-    uint16_t* d_lids = nullptr;         // [I][n] partition-relative ids (partitions <= 65536 points)
     float* d_own = nullptr;             // rows copied in by dcih_append (the index owns these)
     float* d_ukeys = nullptr;           // [I][own_rows] unsorted projections of the rows in d_own
     int64_t own_rows = 0;               // capacity of d_own / d_ukeys in rows
@@ -183,7 +182,6 @@ int release_sorted(dcih_index* h) {
     h->d_skeys = nullptr;
     h->d_sids = nullptr;
     h->d_inv = nullptr;
-    h->d_lids = nullptr;
     h->d_stop_hint = nullptr;
     return 0;
 }
@@ -237,7 +235,7 @@ int ensure_arena(dcih_index* h, int which, size_t bytes) {
 
 // Where the arrays of an index of n points lie inside an arena.
 struct ArenaLayout {
-    size_t keys, ids, inv, lids, hint, total;   // byte offsets, and the size of it all
+    size_t keys, ids, inv, hint, total;         // byte offsets, and the size of it all
     bool small_parts;                           // partitions of at most 65536 points: 16-bit tables exist
 };
 ArenaLayout arena_layout(int I, int64_t n, int block_size) {
@@ -246,15 +244,13 @@ ArenaLayout arena_layout(int I, int64_t n, int block_size) {
     y.small_parts = (n + block_size - 1) / block_size <= 65536;
     const size_t b_keys = align_up(cells * sizeof(float));
     const size_t b_ids = align_up(cells * sizeof(int32_t));
-    const size_t b_inv = y.small_parts ? align_up(cells * sizeof(uint16_t)) : 0;
-    // +16: the traversal reads whole aligned 16-byte chunks, also at the very end
-    const size_t b_lids = y.small_parts ? align_up((cells + 16) * sizeof(uint16_t)) : 0;
+    // +16: the traversal reads whole 16-byte chunks of positions, also at the very end
+    const size_t b_inv = y.small_parts ? align_up((cells + 16) * sizeof(uint16_t)) : 0;
     const size_t b_hint = align_up((size_t)3 * block_size * sizeof(float));   // stop step, promotions at the stop, stops seen
     y.keys = 0;
     y.ids = b_keys;
     y.inv = y.ids + b_ids;
-    y.lids = y.inv + b_inv;
-    y.hint = y.lids + b_lids;
+    y.hint = y.inv + b_inv;
     y.total = y.hint + b_hint;
     return y;
 }
@@ -342,7 +338,6 @@ static int sort_into(dcih_index* h, int which, const float* d_keys, int64_t key_
     float* skeys = (float*)(base + y.keys);
     int32_t* sids = (int32_t*)(base + y.ids);
     uint16_t* inv = y.small_parts ? (uint16_t*)(base + y.inv) : nullptr;
-    uint16_t* lids = y.small_parts ? (uint16_t*)(base + y.lids) : nullptr;
     float* hint = (float*)(base + y.hint);
     // (the table's room is a multiple of 256 bytes, so whole 64-bit words may be cleared)
     int rc = zero_words64(hint, (int64_t)(((size_t)3 * block_size * sizeof(float) + 7) / 8), s);
@@ -350,9 +345,9 @@ static int sort_into(dcih_index* h, int which, const float* d_keys, int64_t key_
         mark(h, DCIH_T_SEGSORT, 0, s);
         if (merge_from > 0)
             rc = segsort_append(h->d_skeys, h->d_sids, merge_from, d_keys, key_stride, I, num_points, block_size,
-                                skeys, sids, inv, lids, d_tmp, s);
+                                skeys, sids, inv, nullptr, d_tmp, s);
         else
-            rc = segsort(d_keys, key_stride, I, num_points, block_size, skeys, sids, inv, lids, d_tmp, s);
+            rc = segsort(d_keys, key_stride, I, num_points, block_size, skeys, sids, inv, nullptr, d_tmp, s);
         mark(h, DCIH_T_SEGSORT, 1, s);
     }
     // like the reference's dci_add, the call returns when the index is complete
@@ -360,7 +355,7 @@ static int sort_into(dcih_index* h, int which, const float* d_keys, int64_t key_
     if (rc == DCIH_OK && se != hipSuccess)
         rc = fail(DCIH_EHIP, std::string("build: ") + hipGetErrorString(se));
     if (rc) return rc;
-    h->d_skeys = skeys; h->d_sids = sids; h->d_inv = inv; h->d_lids = lids; h->d_stop_hint = hint;
+    h->d_skeys = skeys; h->d_sids = sids; h->d_inv = inv; h->d_stop_hint = hint;
     h->cur = which;
     h->d_data = d_data;
     h->n = num_points;
@@ -539,7 +534,7 @@ static int query_impl(dcih_index* h, int dim, int num_queries, const float* d_qu
 
     h->ev_valid[DCIH_T_BATCH] = h->ev_valid[DCIH_T_DENSE] = false;
     QueryArgs a;
-    a.skeys = h->d_skeys; a.sids = h->d_sids; a.inv = h->d_inv; a.lids = h->d_lids; a.data = h->d_data; a.query = d_query;
+    a.skeys = h->d_skeys; a.sids = h->d_sids; a.inv = h->d_inv; a.data = h->d_data; a.query = d_query;
     a.mode = h->traversal; a.item_list = nullptr; a.item_count = nullptr; a.dense = nullptr;
     a.xcds = h->xcds; a.q_first = 0; a.q_count = num_queries;
     a.dense_items = nullptr; a.dense_count = nullptr; a.dense_cap = 0;

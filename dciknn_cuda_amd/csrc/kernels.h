@@ -17,9 +17,10 @@ int project(const float* d_dirs, int num_dirs, const float* d_rows, int64_t num_
 // that is 0).
 size_t segsort_tmp_bytes(int num_indices, int64_t n, int block_size);
 // d_inv: null, or [num_indices][n] receiving each point's position inside its
-// sorted slice (the inverse of d_sids) as a 16-bit value.  d_lids: null, or [num_indices][n]
-// receiving the ids relative to their partition's first point as 16-bit values
-// (only meaningful when a partition holds at most 65536 points).
+// sorted slice (the inverse of d_sids) as a 16-bit value (only meaningful when a partition
+// holds at most 65536 points).  d_lids: null, or [num_indices][n] receiving the ids relative
+// to their partition's first point as 16-bit values (no kernel reads them any more; the
+// index does not keep them).
 int segsort(const float* d_keys, int64_t key_stride, int num_indices, int64_t n, int block_size,
             float* d_skeys, int32_t* d_sids, uint16_t* d_inv, uint16_t* d_lids, void* d_tmp,
             hipStream_t s);
@@ -40,7 +41,6 @@ struct QueryArgs {
     const float* skeys;      // [I][N] sorted projections
     const int32_t* sids;     // [I][N] point ids in the same order
     const uint16_t* inv;     // [I][N] position of every point inside its sorted slice (null if ppb > 65536)
-    const uint16_t* lids;    // [I][N] ids relative to the partition start (null if ppb > 65536)
     const float* data;       // [N][dim]
     const float* query;      // [nq][dim]
     const float* qproj;      // [I][nq]

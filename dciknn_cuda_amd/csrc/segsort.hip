@@ -772,8 +772,8 @@ int segsort(const float* d_keys, int64_t key_stride, int num_indices, int64_t n,
     return 0;
 }
 
-// inv[point] = position of the point inside its sorted slice, from the slice's local ids.
-__global__ __launch_bounds__(512) void slice_inverse_kernel(const uint16_t* __restrict__ lids,
+// inv[point] = position of the point inside its sorted slice, from the slice's sorted ids.
+__global__ __launch_bounds__(512) void slice_inverse_kernel(const int32_t* __restrict__ sids,
                                                             uint16_t* __restrict__ inv, int64_t n, int64_t ppb, int B) {
     extern __shared__ uint16_t pos_of[];
     const int b = (int)(blockIdx.x % B);
@@ -782,7 +782,7 @@ __global__ __launch_bounds__(512) void slice_inverse_kernel(const uint16_t* __re
     const int len = (int)min(ppb, n - off);
     if (len <= 0) return;
     const int64_t base = i * n + off;
-    for (int j = threadIdx.x; j < len; j += blockDim.x) pos_of[lids[base + j]] = (uint16_t)j;
+    for (int j = threadIdx.x; j < len; j += blockDim.x) pos_of[sids[base + j] - (int32_t)off] = (uint16_t)j;
     __syncthreads();
     for (int j = threadIdx.x; j < len; j += blockDim.x) inv[base + j] = pos_of[j];
 }
@@ -850,7 +850,7 @@ int segsort_append(const float* d_old_skeys, const int32_t* d_old_sids, int64_t 
         if (last) break;
     }
     DCIH_HIP(hipGetLastError());
-    // 4. the inverse permutation of every slice from its local ids, turned round in LDS so that
+    // 4. the inverse permutation of every slice from its sorted ids, turned round in LDS so that
     // reads and writes are coalesced (written from the merge it would be a scatter of 2-byte words)
     if (d_inv) {
         const size_t lds = (size_t)ag.p1 * sizeof(uint16_t);
@@ -862,7 +862,7 @@ int segsort_append(const float* d_old_skeys, const int32_t* d_old_sids, int64_t 
         });
         if (rc) return rc;
         hipLaunchKernelGGL(slice_inverse_kernel, dim3((unsigned)((int64_t)num_indices * block_size)), dim3(512), lds, s,
-                           d_lids, d_inv, n1, ag.p1, block_size);
+                           d_sids, d_inv, n1, ag.p1, block_size);
         DCIH_HIP(hipGetLastError());
     }
     return 0;
