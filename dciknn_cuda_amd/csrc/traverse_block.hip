@@ -148,6 +148,13 @@ __global__ __launch_bounds__(NT, MINW) void traverse_block_kernel(QueryArgs a, B
     // cannot rule out (PHASE_END): loads and address arithmetic of the phases after it are then
     // not moved up across it, or out of the epoch loop.  Without the two, the five-workgroup
     // variant keeps 244 bytes per lane in scratch instead of 12 and the kernel runs a quarter slower.
+#define PHASE_FENCE()                                    \
+    do {                                                 \
+        int leave_now = 0;                               \
+        asm volatile("" : "+s"(leave_now));              \
+        if (leave_now) return;                           \
+        fresh_thread_ids();                              \
+    } while (0)
 #define PHASE_END(which)                                 \
     do {                                                 \
         phase(which);                                    \
@@ -503,6 +510,7 @@ __global__ __launch_bounds__(NT, MINW) void traverse_block_kernel(QueryArgs a, B
             }
             __syncthreads();
         }
+        PHASE_FENCE();
         {
             // Eight lanes rank one promotion, so 32 promotions are in flight per
             // workgroup; each lane runs the binary searches of up to three streams in
@@ -632,6 +640,7 @@ __global__ __launch_bounds__(NT, MINW) void traverse_block_kernel(QueryArgs a, B
             for (int j = ne + tid; j < np2; j += NT) events[j] = ~0ull;
             bitonic_sort_u64(events, np2);
         }
+        PHASE_FENCE();
         if (ne <= kWave && wave == 0) {
             // Up to one event per lane: the walk below is the same as the serial one after
             // it, but reads steps and flags from registers (lane reads, ballots) instead of
@@ -804,6 +813,7 @@ __global__ __launch_bounds__(NT, MINW) void traverse_block_kernel(QueryArgs a, B
             hand_to_dense();
             return;
         }
+        PHASE_FENCE();
         bool mine_exhausted = true;     // every wavefront looks at all S <= 128 streams, a lane at two
         for (int s = lane; s < S; s += kWave) mine_exhausted = mine_exhausted && s_c[s] >= s_ns[s];
         if (__all(mine_exhausted)) break;     // H was unbounded: everything has been replayed
@@ -897,6 +907,7 @@ __global__ __launch_bounds__(NT, MINW) void traverse_block_kernel(QueryArgs a, B
 constexpr int kBlockThreads = 256;
 
 #undef PHASE_END
+#undef PHASE_FENCE
 
 }  // namespace
 
