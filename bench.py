@@ -378,6 +378,9 @@ def main():
         roofline["traffic_fetch_bytes"], roofline["traffic_write_bytes"] = prof["fetch_bytes"], prof["write_bytes"]
         if "valu_issue_frac" in prof:
             roofline["valu_issue_frac_profiled"] = prof["valu_issue_frac"]
+        if "l2_read_bytes" in prof:     # TCP_TCC_READ_REQ_sum x 128 B in the counter run
+            roofline["l2_read_bytes_profiled"] = prof["l2_read_bytes"]
+            roofline["l2_frac_profiled"] = prof["l2_frac"]
 
     build_bytes_proj = 4.0 * new_rows * (dim + I)
     build_bytes_sort = 12.0 * N * I
