@@ -211,3 +211,19 @@ def test_bench_refuses_more_than_one_gpu():
                        capture_output=True, text=True, timeout=120)
     assert r.returncode != 0
     assert "ONE GPU" in r.stderr and r.stdout.strip() == ""
+
+
+def test_traffic_table_names_commits_of_this_history():
+    """Every row of profiles/hbm_traffic.json (the counter runs bench.py's `traffic` comes from) names
+    the setting it was taken at and a commit that exists in this repository's history."""
+    import json
+    import subprocess
+    runs = json.load(open(os.path.join(ROOT, "profiles", "hbm_traffic.json")))["runs"]
+    assert runs
+    have_git = os.path.isdir(os.path.join(ROOT, ".git"))
+    for r in runs:
+        assert {"config", "bs", "ts", "outer", "queries", "kernel", "commit"} <= set(r), r
+        assert re.fullmatch(r"[0-9a-f]{7,40}", r["commit"]), r["commit"]
+        if have_git:
+            kind = subprocess.run(["git", "-C", ROOT, "cat-file", "-t", r["commit"]], capture_output=True, text=True)
+            assert kind.stdout.strip() == "commit", r["commit"]
