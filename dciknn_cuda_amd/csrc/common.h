@@ -54,26 +54,68 @@ __host__ __device__ inline float ord2f(uint32_t u) {
 }
 
 #if defined(__HIPCC__)
+// ---- exchanges between the lanes of a wavefront -----------------------------------
+// The value lane (l ^ O) holds, O a power of two below 64, without an address register: within
+// quads by DPP, within 32 lanes by ds_swizzle with an immediate pattern, across the halves by
+// v_permlane32_swap.  (__shfl_xor computes a byte address per lane from the lane number, which
+// the compiler then keeps alive -- or spills -- across a whole kernel.)
+template <int O>
+__device__ inline uint32_t lane_xor_u32(uint32_t v) {
+    static_assert(O == 1 || O == 2 || O == 4 || O == 8 || O == 16 || O == 32, "one lane bit");
+    if constexpr (O == 1) {
+        return (uint32_t)__builtin_amdgcn_mov_dpp((int)v, 0xB1, 0xf, 0xf, true);      // quad_perm [1,0,3,2]
+    } else if constexpr (O == 2) {
+        return (uint32_t)__builtin_amdgcn_mov_dpp((int)v, 0x4E, 0xf, 0xf, true);      // quad_perm [2,3,0,1]
+    } else if constexpr (O == 32) {
+        // after the swap, [0] holds in its upper half what the lower half of v held, and [1] in its
+        // lower half what the upper half held
+        const auto r = __builtin_amdgcn_permlane32_swap(v, v, false, false);
+        uint32_t out;
+        asm("v_cndmask_b32 %0, %1, %2, %3" : "=v"(out) : "v"(r[1]), "v"(r[0]), "s"(0xffffffff00000000ull));
+        return out;
+    } else {
+        return (uint32_t)__builtin_amdgcn_ds_swizzle((int)v, (O << 10) | 0x1f);       // xor mask, and mask 0x1f
+    }
+}
+template <int O> __device__ inline int lane_xor(int v) { return (int)lane_xor_u32<O>((uint32_t)v); }
+template <int O> __device__ inline uint32_t lane_xor(uint32_t v) { return lane_xor_u32<O>(v); }
+template <int O> __device__ inline float lane_xor(float v) {
+    return __builtin_bit_cast(float, lane_xor_u32<O>(__builtin_bit_cast(uint32_t, v)));
+}
+template <int O> __device__ inline unsigned long long lane_xor(unsigned long long v) {
+    return ((unsigned long long)lane_xor_u32<O>((uint32_t)(v >> 32)) << 32) | lane_xor_u32<O>((uint32_t)v);
+}
+
 // ---- wavefront (64-lane) reductions ----------------------------------------
+// (levels in the order 32, 16, .., 1: the traversal kernels rely on this order for equal bits)
 __device__ inline float wave_sum(float v) {
-#pragma unroll
-    for (int o = 32; o > 0; o >>= 1) v += __shfl_xor(v, o, kWave);
+    v += lane_xor<32>(v); v += lane_xor<16>(v); v += lane_xor<8>(v);
+    v += lane_xor<4>(v); v += lane_xor<2>(v); v += lane_xor<1>(v);
     return v;
 }
 __device__ inline uint32_t wave_min_u32(uint32_t v) {
-#pragma unroll
-    for (int o = 32; o > 0; o >>= 1) {
-        uint32_t w = (uint32_t)__shfl_xor((int)v, o, kWave);
-        v = w < v ? w : v;
-    }
+    v = min(v, lane_xor<32>(v)); v = min(v, lane_xor<16>(v)); v = min(v, lane_xor<8>(v));
+    v = min(v, lane_xor<4>(v)); v = min(v, lane_xor<2>(v)); v = min(v, lane_xor<1>(v));
+    return v;
+}
+__device__ inline uint32_t wave_sum_u32(uint32_t v) {
+    v += lane_xor<32>(v); v += lane_xor<16>(v); v += lane_xor<8>(v);
+    v += lane_xor<4>(v); v += lane_xor<2>(v); v += lane_xor<1>(v);
+    return v;
+}
+__device__ inline int wave_max_i32(int v) {
+    v = max(v, lane_xor<32>(v)); v = max(v, lane_xor<16>(v)); v = max(v, lane_xor<8>(v));
+    v = max(v, lane_xor<4>(v)); v = max(v, lane_xor<2>(v)); v = max(v, lane_xor<1>(v));
     return v;
 }
 __device__ inline unsigned long long wave_max_u64(unsigned long long v) {
-#pragma unroll
-    for (int o = 32; o > 0; o >>= 1) {
-        unsigned long long w = __shfl_xor(v, o, kWave);
-        v = w > v ? w : v;
-    }
+    unsigned long long w;
+    w = lane_xor<32>(v); v = w > v ? w : v;
+    w = lane_xor<16>(v); v = w > v ? w : v;
+    w = lane_xor<8>(v); v = w > v ? w : v;
+    w = lane_xor<4>(v); v = w > v ? w : v;
+    w = lane_xor<2>(v); v = w > v ? w : v;
+    w = lane_xor<1>(v); v = w > v ? w : v;
     return v;
 }
 __device__ inline int lane_id() { return (int)(threadIdx.x & (kWave - 1)); }
@@ -87,8 +129,8 @@ __device__ inline int lane_id() { return (int)(threadIdx.x & (kWave - 1)); }
 // interleaves the reads of independent rows.
 template <int R>
 __device__ inline void wave_row_dists(const float* const (&rows)[R], const float* q, int dim,
-                                      bool vec4, float (&dist)[R]) {
-    const int lane = lane_id();
+                                      bool vec4, float (&dist)[R], int lane = -1) {
+    if (lane < 0) lane = lane_id();      // (callers that keep their own lane number pass it)
     float acc[R];
 #pragma unroll
     for (int r = 0; r < R; r++) acc[r] = 0.f;
@@ -169,20 +211,27 @@ __device__ inline bool rows_vec4(const float* data, int dim) {
 
 // In-place ascending bitonic sort of `n` (a power of two) 64-bit words in LDS
 // by all threads of the block (which has at least one full wavefront).
-__device__ inline void bitonic_sort_u64(unsigned long long* s, int n) {
+template <int SIZE, int STRIDE>
+__device__ inline void bitonic_wave_steps(unsigned long long& v, int lane, int n) {
+    if (SIZE <= n) {       // (same on every lane)
+        const unsigned long long o = lane_xor<STRIDE>(v);
+        const bool keep_min = ((lane & STRIDE) == 0) == ((lane & SIZE) == 0);
+        v = keep_min ? (v < o ? v : o) : (v > o ? v : o);
+    }
+    if constexpr (STRIDE > 1) bitonic_wave_steps<SIZE, STRIDE / 2>(v, lane, n);
+    else if constexpr (SIZE < kWave) bitonic_wave_steps<SIZE * 2, SIZE>(v, lane, n);
+}
+// `tid` is the caller's thread number (a caller that hides its thread number from the
+// compiler between phases passes its own copy).
+__device__ inline void bitonic_sort_u64(unsigned long long* s, int n, int tid = -1) {
+    if (tid < 0) tid = (int)threadIdx.x;
     if (n <= kWave) {
         // one wavefront sorts in registers with lane exchanges: no barrier per stage
         __syncthreads();
-        if (threadIdx.x < kWave) {
-            const int lane = (int)threadIdx.x;
+        if (tid < kWave) {
+            const int lane = tid;
             unsigned long long v = lane < n ? s[lane] : ~0ull;
-            for (int size = 2; size <= n; size <<= 1) {
-                for (int stride = size >> 1; stride > 0; stride >>= 1) {
-                    const unsigned long long o = __shfl_xor(v, stride, kWave);
-                    const bool keep_min = ((lane & stride) == 0) == ((lane & size) == 0);
-                    v = keep_min ? (v < o ? v : o) : (v > o ? v : o);
-                }
-            }
+            bitonic_wave_steps<2, 1>(v, lane, n);
             if (lane < n) s[lane] = v;
         }
         __syncthreads();
@@ -191,7 +240,7 @@ __device__ inline void bitonic_sort_u64(unsigned long long* s, int n) {
     for (int size = 2; size <= n; size <<= 1) {
         for (int stride = size >> 1; stride > 0; stride >>= 1) {
             __syncthreads();
-            for (int t = threadIdx.x; t < (n >> 1); t += blockDim.x) {
+            for (int t = tid; t < (n >> 1); t += blockDim.x) {
                 int lo = 2 * t - (t & (stride - 1));
                 int hi = lo + stride;
                 bool up = (lo & size) == 0;

@@ -48,7 +48,8 @@ constexpr int kMaxEpochs = 100000;
 
 enum Misc {   // 32-bit scalars shared by the workgroup
     kPromoCount = 0, kEventCount, kAccCount, kFail, kStop, kC0, kStopStepLo, kStopStepHi,
-    kArmedLo, kArmedHi, kScannedLo, kScannedHi, kArmed, kNumCand, kTopN, kProbes, kHintSteps, kHintPromos, kMiscWords
+    kArmedLo, kArmedHi, kScannedLo, kScannedHi, kArmed, kNumCand, kTopN, kProbes, kHintSteps, kHintPromos,
+    kFirstJump, kPromoAimBits, kInvLBits, kMiscWords
 };
 
 struct BlockLayout {
@@ -277,10 +278,17 @@ __global__ __launch_bounds__(NT, MINW) void traverse_block_kernel(QueryArgs a, B
     {
         int first = 4;           // (every wavefront reduces the S <= 128 stream lengths on its own)
         for (int s = lane; s < S; s += kWave) first = max(first, s_ns[s] / 128);
-        for (int o = kWave / 2; o > 0; o >>= 1) first = max(first, __shfl_xor(first, o, kWave));
+        first = wave_max_i32(first);
         if (hint > 0.0f) first = max(first, (int)(kHintFirst * hint / (float)(2 * a.L)));
         if (tid < S) s_stride[tid] = first;
         if (tid < a.M) s_Kprev[tid] = 0;
+        // (the later epochs' sizing reads these back from LDS instead of keeping them in registers --
+        //  in scratch, in the tight variants -- across all phases)
+        if (tid == 0) {
+            misc[kFirstJump] = __builtin_bit_cast(uint32_t, kHintFirst);
+            misc[kPromoAimBits] = __builtin_bit_cast(uint32_t, kPromoAim);
+            misc[kInvLBits] = __builtin_bit_cast(uint32_t, inv_L);
+        }
     }
     __syncthreads();
     PHASE_END(0);
@@ -389,10 +397,6 @@ __global__ __launch_bounds__(NT, MINW) void traverse_block_kernel(QueryArgs a, B
             atomicOr(&marked[m * y.seen_words + (local >> 5)], 1u << (local & 31u));
         }
     };
-    // index entries the scans looked at (same on every thread)
-    const unsigned long long scan_entries = (unsigned long long)n * (unsigned long long)I;
-
-    unsigned long long scanned = 0;      // entries scanned so far (same on every thread)
     bool shrunk = false;        // the previous epoch was undone
     bool undone_once = false;   // some epoch of this item was undone
     int epoch = 0;
@@ -469,7 +473,7 @@ __global__ __launch_bounds__(NT, MINW) void traverse_block_kernel(QueryArgs a, B
 
         // ---- 3. the points whose L windows are now all consumed ---------------------
         scan_epoch();
-        scanned += scan_entries;
+        if (a.counters && tid == 0) atomicAdd(&misc[kScannedLo], 1u);      // scans so far, each over n * I index entries
         __syncthreads();
         PHASE_END(3);
         const uint32_t np = misc[kPromoCount];
@@ -544,15 +548,20 @@ __global__ __launch_bounds__(NT, MINW) void traverse_block_kernel(QueryArgs a, B
                     const uint32_t bits = __builtin_bit_cast(uint32_t, fabsf(key[kp] - s_qp[i]));
                     if (w_h < 0 || bits >= w_bits) { w_bits = bits; w_h = h; w_side = side; w_j = j; w_t = t; }
                 }
-                for (int o = kGroup / 2; o > 0; o >>= 1) {
-                    const uint32_t ob = (uint32_t)__shfl_xor((int)w_bits, o, kGroup);
-                    const int oh = __shfl_xor(w_h, o, kGroup);
-                    const int os = __shfl_xor(w_side, o, kGroup);
-                    const int oj = __shfl_xor(w_j, o, kGroup);
-                    const int ot = __shfl_xor(w_t, o, kGroup);
+                auto farthest_of_two = [&](auto width) {      // (lane exchanges by immediate patterns: no address registers)
+                    constexpr int O = decltype(width)::value;
+                    const uint32_t ob = lane_xor<O>(w_bits);
+                    const int oh = lane_xor<O>(w_h);
+                    const int os = lane_xor<O>(w_side);
+                    const int oj = lane_xor<O>(w_j);
+                    const int ot = lane_xor<O>(w_t);
                     const bool take = oh >= 0 && (w_h < 0 || ob > w_bits || (ob == w_bits && oh > w_h));
                     if (take) { w_bits = ob; w_h = oh; w_side = os; w_j = oj; w_t = ot; }
-                }
+                };
+                static_assert(kGroup == 8, "three exchange levels");
+                farthest_of_two(std::integral_constant<int, 4>());
+                farthest_of_two(std::integral_constant<int, 2>());
+                farthest_of_two(std::integral_constant<int, 1>());
                 // rank of that window = windows of the composite ordered before it
                 uint32_t rank = 0;
                 for (int s0 = gl; s0 < 2 * a.L; s0 += kGroup * kPerLane) {
@@ -611,7 +620,7 @@ __global__ __launch_bounds__(NT, MINW) void traverse_block_kernel(QueryArgs a, B
 #pragma unroll
                     for (int u = 0; u < kPerLane; u++) rank += (uint32_t)lo[u];
                 }
-                for (int o = kGroup / 2; o > 0; o >>= 1) rank += (uint32_t)__shfl_xor((int)rank, o, kGroup);
+                rank += lane_xor<4>(rank); rank += lane_xor<2>(rank); rank += lane_xor<1>(rank);
                 if (gl == 0) {
                     const uint32_t slot = atomicAdd(&misc[kEventCount], 1u);
                     if (slot < (uint32_t)y.event_cap) events[slot] = pack_event(rank, m, w_t == 0, local);
@@ -638,7 +647,7 @@ __global__ __launch_bounds__(NT, MINW) void traverse_block_kernel(QueryArgs a, B
             int np2 = 2;
             while (np2 < ne) np2 <<= 1;
             for (int j = ne + tid; j < np2; j += NT) events[j] = ~0ull;
-            bitonic_sort_u64(events, np2);
+            bitonic_sort_u64(events, np2, tid);
         }
         PHASE_FENCE();
         if (ne <= kWave && wave == 0) {
@@ -787,7 +796,7 @@ __global__ __launch_bounds__(NT, MINW) void traverse_block_kernel(QueryArgs a, B
                 const int64_t pt1 = c2 < batch ? off + acc[done + c2] : pt0;
                 const float* const rows2[2] = {a.data + pt0 * a.dim, a.data + pt1 * a.dim};
                 float d2[2];
-                wave_row_dists<2>(rows2, s_q, a.dim, vec4, d2);
+                wave_row_dists<2>(rows2, s_q, a.dim, vec4, d2, lane);
                 if (lane == 0) {
                     sortbuf[topn + c] = ((unsigned long long)__builtin_bit_cast(uint32_t, d2[0]) << 32) | (uint32_t)pt0;
                     if (c2 < batch)
@@ -797,7 +806,7 @@ __global__ __launch_bounds__(NT, MINW) void traverse_block_kernel(QueryArgs a, B
             int np2 = 2;
             while (np2 < topn + batch) np2 <<= 1;
             for (int j = topn + batch + tid; j < np2; j += NT) sortbuf[j] = ~0ull;
-            bitonic_sort_u64(sortbuf, np2);
+            bitonic_sort_u64(sortbuf, np2, tid);
             if (tid == 0) misc[kTopN] = (uint32_t)min(a.kcap, topn + batch);
             done += batch;
             __syncthreads();
@@ -823,17 +832,22 @@ __global__ __launch_bounds__(NT, MINW) void traverse_block_kernel(QueryArgs a, B
                 if (s_K[m] >= kmax) { kmax = s_K[m]; dk_lead = max(1u, s_K[m] - s_Kprev[m]); }
             // where to land next (steps per composite): just past the stop step once
             // c0 >= k; else by the hint; else twice the last stride
+            const float hint_here = __builtin_bit_cast(float, misc[kHintSteps]);
+            const float first_jump = __builtin_bit_cast(float, misc[kFirstJump]);
+            const float aim = __builtin_bit_cast(float, misc[kPromoAimBits]);
+            const float inv_L_here = __builtin_bit_cast(float, misc[kInvLBits]);
+            const float S_f = (float)S;
             float k_target = (float)kmax + 2.0f * (float)dk_lead;
             const float need = (float)(a.stop_at > 0 ? a.stop_at : 1);
             if (misc[kArmed]) {
                 const float t_armed = (float)(((unsigned long long)misc[kArmedHi] << 32) | misc[kArmedLo]);
-                k_target = fmaxf(t_armed + 1.0f, need) + (float)S;
-            } else if (hint > 0.0f) {
+                k_target = fmaxf(t_armed + 1.0f, need) + S_f;
+            } else if (hint_here > 0.0f) {
                 const float so_far = (float)max(1u, misc[kNumCand] + misc[kEventCount]);   // promotions up to here
-                const float grow = fminf(kHintGrow, fast_pow(1.0f + kPromoAim / so_far, inv_L));
-                k_target = (float)kmax < 0.9f * kHintFirst * hint ? kHintFirst * hint : grow * (float)kmax + (float)S;
+                const float grow = fminf(kHintGrow, fast_pow(1.0f + aim / so_far, inv_L_here));
+                k_target = (float)kmax < 0.9f * first_jump * hint_here ? first_jump * hint_here : grow * (float)kmax + S_f;
             }
-            k_target = fminf(k_target, 2.0f * (float)kmax + 16.0f * (float)S);
+            k_target = fminf(k_target, 2.0f * (float)kmax + 16.0f * S_f);
             if (shrunk) k_target = fminf(k_target, (float)kmax + 2.0f * (float)dk_lead);
             shrunk = false;       // the epoch after an undo was accepted: back to aimed epochs
             __syncthreads();
@@ -876,9 +890,8 @@ __global__ __launch_bounds__(NT, MINW) void traverse_block_kernel(QueryArgs a, B
     const int topn = (int)misc[kTopN];
     for (int j = tid; j < a.kcap; j += NT) part_out[j] = j < topn ? sortbuf[j] : ~0ull;
     if (a.counters) {
-        for (int o = 32; o > 0; o >>= 1) probes += (uint32_t)__shfl_xor((int)probes, o, kWave);
+        probes = wave_sum_u32(probes);
         if (lane == 0) atomicAdd(&misc[kProbes], probes);
-        if (tid == 0) { misc[kScannedLo] = (uint32_t)scanned; misc[kScannedHi] = (uint32_t)(scanned >> 32); }
         __syncthreads();
         if (tid == 0) {
             unsigned long long steps;   // outer steps the loop would have run (:458, :598-609)
@@ -895,7 +908,7 @@ __global__ __launch_bounds__(NT, MINW) void traverse_block_kernel(QueryArgs a, B
             } else {
                 steps = min(bound, maxw + 1);
             }
-            const unsigned long long st = ((unsigned long long)misc[kScannedHi] << 32) | misc[kScannedLo];
+            const unsigned long long st = (unsigned long long)misc[kScannedLo] * (unsigned long long)n * (unsigned long long)I;
             atomicAdd(&a.counters[(int64_t)qi * 4 + 0], st);
             atomicAdd(&a.counters[(int64_t)qi * 4 + 1], (unsigned long long)misc[kNumCand]);
             atomicAdd(&a.counters[(int64_t)qi * 4 + 2], (unsigned long long)misc[kProbes]);
