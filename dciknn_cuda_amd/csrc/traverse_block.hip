@@ -49,7 +49,7 @@ constexpr int kMaxEpochs = 100000;
 enum Misc {   // 32-bit scalars shared by the workgroup
     kPromoCount = 0, kEventCount, kAccCount, kFail, kStop, kC0, kStopStepLo, kStopStepHi,
     kArmedLo, kArmedHi, kScannedLo, kScannedHi, kArmed, kNumCand, kTopN, kProbes, kHintSteps, kHintPromos,
-    kFirstJump, kPromoAimBits, kInvLBits, kMiscWords
+    kFirstJump, kPromoAimBits, kInvLBits, kNeedBits, kItem, kMiscWords
 };
 
 struct BlockLayout {
@@ -203,13 +203,14 @@ __global__ __launch_bounds__(NT, MINW) void traverse_block_kernel(QueryArgs a, B
         if (threadIdx.x == 0) {
             const int x = (int)(blockIdx.x % a.xcds);
             const uint32_t sl = atomicAdd(&a.dense_count[x], 1u);
-            a.dense_items[(int64_t)x * a.dense_cap + sl] = (int32_t)item;
+            a.dense_items[(int64_t)x * a.dense_cap + sl] = (int32_t)misc[kItem];      // (read back: no register held for it)
         }
     };
     // usual stop step and promotions at the stop: read by one thread, because other workgroups
     // are updating them and every thread must decide alike
     if (threadIdx.x < kMiscWords) misc[threadIdx.x] = 0;
     __syncthreads();
+    if (threadIdx.x == 0) misc[kItem] = (uint32_t)item;
     if (threadIdx.x == 0 && a.stop_hint) {
         float steps, promotions;
         usual_stop(a.stop_hint, a.B, b, steps, promotions);
@@ -288,6 +289,7 @@ __global__ __launch_bounds__(NT, MINW) void traverse_block_kernel(QueryArgs a, B
             misc[kFirstJump] = __builtin_bit_cast(uint32_t, kHintFirst);
             misc[kPromoAimBits] = __builtin_bit_cast(uint32_t, kPromoAim);
             misc[kInvLBits] = __builtin_bit_cast(uint32_t, inv_L);
+            misc[kNeedBits] = __builtin_bit_cast(uint32_t, (float)(a.stop_at > 0 ? a.stop_at : 1));
         }
     }
     __syncthreads();
@@ -838,7 +840,7 @@ __global__ __launch_bounds__(NT, MINW) void traverse_block_kernel(QueryArgs a, B
             const float inv_L_here = __builtin_bit_cast(float, misc[kInvLBits]);
             const float S_f = (float)S;
             float k_target = (float)kmax + 2.0f * (float)dk_lead;
-            const float need = (float)(a.stop_at > 0 ? a.stop_at : 1);
+            const float need = __builtin_bit_cast(float, misc[kNeedBits]);
             if (misc[kArmed]) {
                 const float t_armed = (float)(((unsigned long long)misc[kArmedHi] << 32) | misc[kArmedLo]);
                 k_target = fmaxf(t_armed + 1.0f, need) + S_f;
