@@ -126,6 +126,9 @@ struct dcih_index {
     float* d_skeys = nullptr;           // [I][n]
     int32_t* d_sids = nullptr;          // [I][n]
     uint16_t* d_inv = nullptr;          // [I][n] position of each point in its sorted slice (partitions <= 65536 points)
+    uint16_t* d_rpos = nullptr;         // [I][n] the same, in the order of each composite's first simple index (room kept by the
+                                        // build, filled by the first query that runs the batch traversal kernel)
+    int rpos_ready = 0;
     float* d_own = nullptr;             // rows copied in by dcih_append (the index owns these)
     float* d_ukeys = nullptr;           // [I][own_rows] unsorted projections of the rows in d_own
     int64_t own_rows = 0;               // capacity of d_own / d_ukeys in rows
@@ -182,6 +185,8 @@ int release_sorted(dcih_index* h) {
     h->d_skeys = nullptr;
     h->d_sids = nullptr;
     h->d_inv = nullptr;
+    h->d_rpos = nullptr;
+    h->rpos_ready = 0;
     h->d_stop_hint = nullptr;
     return 0;
 }
@@ -235,7 +240,7 @@ int ensure_arena(dcih_index* h, int which, size_t bytes) {
 
 // Where the arrays of an index of n points lie inside an arena.
 struct ArenaLayout {
-    size_t keys, ids, inv, hint, total;         // byte offsets, and the size of it all
+    size_t keys, ids, inv, rpos, hint, total;   // byte offsets, and the size of it all
     bool small_parts;                           // partitions of at most 65536 points: 16-bit tables exist
 };
 ArenaLayout arena_layout(int I, int64_t n, int block_size) {
@@ -250,7 +255,8 @@ ArenaLayout arena_layout(int I, int64_t n, int block_size) {
     y.keys = 0;
     y.ids = b_keys;
     y.inv = y.ids + b_ids;
-    y.hint = y.inv + b_inv;
+    y.rpos = y.inv + b_inv;
+    y.hint = y.rpos + b_inv;
     y.total = y.hint + b_hint;
     return y;
 }
@@ -356,6 +362,8 @@ static int sort_into(dcih_index* h, int which, const float* d_keys, int64_t key_
         rc = fail(DCIH_EHIP, std::string("build: ") + hipGetErrorString(se));
     if (rc) return rc;
     h->d_skeys = skeys; h->d_sids = sids; h->d_inv = inv; h->d_stop_hint = hint;
+    h->d_rpos = y.small_parts ? (uint16_t*)(base + y.rpos) : nullptr;
+    h->rpos_ready = 0;
     h->cur = which;
     h->d_data = d_data;
     h->n = num_points;
@@ -535,6 +543,7 @@ static int query_impl(dcih_index* h, int dim, int num_queries, const float* d_qu
     h->ev_valid[DCIH_T_BATCH] = h->ev_valid[DCIH_T_DENSE] = false;
     QueryArgs a;
     a.skeys = h->d_skeys; a.sids = h->d_sids; a.inv = h->d_inv; a.data = h->d_data; a.query = d_query;
+    a.rpos = h->d_rpos; a.rpos_ready = &h->rpos_ready;
     a.mode = h->traversal; a.item_list = nullptr; a.item_count = nullptr; a.dense = nullptr;
     a.xcds = h->xcds; a.q_first = 0; a.q_count = num_queries;
     a.dense_items = nullptr; a.dense_count = nullptr; a.dense_cap = 0;

@@ -37,10 +37,19 @@ int segsort_append(const float* d_old_skeys, const int32_t* d_old_sids, int64_t 
                    float* d_skeys, int32_t* d_sids, uint16_t* d_inv, uint16_t* d_lids, void* d_tmp,
                    hipStream_t s);
 
+// rpos (above inv's layout, [I][n] 16-bit values): rpos[i][e] = inv[i][sids[first(i)][e]], first(i) = the first simple
+// index of i's composite; the rows of the first simple indices themselves are left alone (the identity).
+int fill_positions_by_first(const int32_t* d_sids, const uint16_t* d_inv, uint16_t* d_rpos, int64_t n, int M, int L,
+                            hipStream_t s);
+
 struct QueryArgs {
     const float* skeys;      // [I][N] sorted projections
     const int32_t* sids;     // [I][N] point ids in the same order
     const uint16_t* inv;     // [I][N] position of every point inside its sorted slice (null if ppb > 65536)
+    const uint16_t* rpos;    // [I][N] the same positions in the order of the composite's FIRST simple index: entry s of a
+                             // slice is the position, in this simple index, of the point that stands at place s of the
+                             // first one's slice (null if ppb > 65536; filled on the first use, see fill_positions_by_first)
+    int* rpos_ready;         // host flag of the index: rpos has been filled
     const float* data;       // [N][dim]
     const float* query;      // [nq][dim]
     const float* qproj;      // [I][nq]

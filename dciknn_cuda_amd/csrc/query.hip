@@ -413,6 +413,11 @@ int query(const QueryArgs& a_in, hipStream_t s, hipEvent_t* ev, bool* ran) {
     a.item_count = nullptr;
     if (use_block || a.mode == 3) {
         if (use_block) {
+            if (a.rpos_ready && !*a.rpos_ready) {      // the first batch traversal over this index
+                const int rc = fill_positions_by_first(a.sids, a.inv, const_cast<uint16_t*>(a.rpos), a.N, a.M, a.L, s);
+                if (rc) return rc;
+                *a.rpos_ready = 1;
+            }
             const int rc = query_block(a, s);
             if (rc) return rc;
             if (ev) (void)hipEventRecord(ev[1], s);

@@ -772,6 +772,40 @@ int segsort(const float* d_keys, int64_t key_stride, int num_indices, int64_t n,
     return 0;
 }
 
+// The positions of every point in simple index i, in the order of the slice of the first simple index r of
+// i's composite: the batch traversal scans them for the points that stand inside the first index's visited run.
+// Point ids of a partition lie in the partition, so the gather stays inside one slice of inv (L1 / L2).
+__global__ __launch_bounds__(256) void positions_by_first_kernel(const int32_t* __restrict__ sids,
+                                                                 const uint16_t* __restrict__ inv,
+                                                                 uint16_t* __restrict__ rpos, int64_t n, int L) {
+    const int m = (int)(blockIdx.y / (L - 1));
+    const int h = 1 + (int)(blockIdx.y % (L - 1));
+    const int64_t r = (int64_t)m * L, i = r + h;
+    const int64_t e0 = ((int64_t)blockIdx.x * 256 + threadIdx.x) * 4;
+    if (e0 >= n) return;
+    if (e0 + 4 <= n && (n & 3) == 0) {       // four at a time: one 16-byte read of ids, one 8-byte write
+        typedef int v4i __attribute__((ext_vector_type(4)));
+        typedef uint16_t v4h __attribute__((ext_vector_type(4)));
+        const v4i p = *reinterpret_cast<const v4i*>(sids + r * n + e0);
+        v4h o;
+        o.x = inv[i * n + p.x]; o.y = inv[i * n + p.y]; o.z = inv[i * n + p.z]; o.w = inv[i * n + p.w];
+        *reinterpret_cast<v4h*>(rpos + i * n + e0) = o;
+    } else {
+        for (int64_t e = e0; e < min(n, e0 + 4); e++) rpos[i * n + e] = inv[i * n + sids[r * n + e]];
+    }
+}
+
+int fill_positions_by_first(const int32_t* d_sids, const uint16_t* d_inv, uint16_t* d_rpos, int64_t n, int M, int L,
+                            hipStream_t s) {
+    if (L < 2 || n <= 0) return 0;
+    const int64_t bx = (n + 1023) / 1024, by = (int64_t)M * (L - 1);
+    if (bx > 0x7fffffffLL || by > 65535) return fail(-1, "fill_positions_by_first: grid too large");
+    hipLaunchKernelGGL(positions_by_first_kernel, dim3((unsigned)bx, (unsigned)by), dim3(256), 0, s,
+                       d_sids, d_inv, d_rpos, n, L);
+    DCIH_HIP(hipGetLastError());
+    return 0;
+}
+
 // inv[point] = position of the point inside its sorted slice, from the slice's sorted ids.
 __global__ __launch_bounds__(512) void slice_inverse_kernel(const int32_t* __restrict__ sids,
                                                             uint16_t* __restrict__ inv, int64_t n, int64_t ppb, int B) {

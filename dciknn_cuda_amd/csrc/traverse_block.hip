@@ -307,22 +307,21 @@ __global__ __launch_bounds__(NT, MINW) void traverse_block_kernel(QueryArgs a, B
     // positions [lo_i, hi_i) of its sorted slice (the left stream's windows end at the query
     // position, the right stream's start there), so composite m has visited a point in all of
     // its L simple indices exactly when the point's position lies in that run in every one of
-    // them.  Every thread takes eight consecutive points at a time: their positions in one
-    // simple index are ONE 16-byte read of the inverse permutation, and per pair of points
+    // them.  Only the points inside the run of the composite's FIRST simple index can qualify,
+    // and a.rpos holds every point's positions in the order of that slice: the scan walks the
+    // first index's run and tests the other L - 1 positions of the points standing there.
+    // Every thread takes eight consecutive places at a time: the positions in one simple
+    // index of the points standing there are ONE 16-byte read, and per pair of points
     // membership costs three packed 16-bit instructions: pos - lo (wrapping), minus
     // (length - 1) with unsigned saturation -- zero exactly when lo <= pos < hi -- and a
-    // running maximum over the simple indices, which ends at zero for the points inside all L
+    // running maximum over the simple indices, which ends at zero for the points inside all
     // runs.  Those not yet promoted under m in an earlier epoch (one bit per point and
     // composite) go to the promotion list.  No state is left behind: an epoch that turns out
-    // too large is simply dropped.  The loop reads L * n positions per composite whatever the
-    // bound, four simple indices' reads in flight per thread.
+    // too large is simply dropped.  The loop reads (L - 1) positions per place of the run, four
+    // simple indices' reads in flight per thread.
     typedef uint16_t u16x2 __attribute__((ext_vector_type(2)));
     typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
     typedef __attribute__((address_space(1))) const u32x4 g_u32x4;
-    // chunks of eight points start where the slices' reads are 16-byte aligned, if the slices of
-    // all simple indices can be aligned together (N a multiple of 8); else reads are unaligned
-    const int chunk_shift = (a.N & 7) == 0 ? (int)(off & 7) : 0;
-    const int nchunks = (n + chunk_shift + 7) >> 3;
     auto scan_epoch = [&]() {
         if (tid < a.M) s_noscan[tid] = 0;
         __syncthreads();
@@ -336,31 +335,46 @@ __global__ __launch_bounds__(NT, MINW) void traverse_block_kernel(QueryArgs a, B
             if (hi <= lo) s_noscan[tid / a.L] = 1;
         }
         __syncthreads();
+        unsigned long long looked_at = 0;      // index entries read (same on every thread)
         for (int m = 0; m < a.M; m++) {
             if (s_noscan[m]) continue;
-            const uint16_t* inv_m = a.inv + (int64_t)m * a.L * a.N + off - chunk_shift;
+            const int64_t first_row = (int64_t)m * a.L * a.N + off;     // the composite's first simple index, this partition
             const uint32_t* lo2 = s_lo2 + m * a.L;
             const uint32_t* lm2 = s_lm2 + m * a.L;
             const uint32_t* marked_m = marked + m * y.seen_words;
+            // the first index's run, in chunks of eight places that start where the reads are 16-byte
+            // aligned, if the slices of all simple indices can be aligned together (N a multiple of
+            // 8); else reads are unaligned
+            const int run_lo = (int)(lo2[0] & 0xffffu), run_hi = run_lo + (int)(lm2[0] & 0xffffu) + 1;
+            const int chunk_shift = (a.N & 7) == 0 ? (int)((off + run_lo) & 7) : 0;
+            const int start = run_lo - chunk_shift;
+            const int nchunks = (run_hi - start + 7) >> 3;
+            looked_at += (unsigned long long)nchunks * 8ull * (unsigned long long)(a.L - 1);
+            const uint16_t* rp = a.rpos + first_row + start;
             for (int c = tid; c < nchunks; c += NT) {
-                const int first = 8 * c - chunk_shift;      // partition-relative id of the chunk's first point
+                const int first = start + 8 * c;            // place in the first index's slice of the chunk's first point
                 u16x2 worst[4];
 #pragma unroll
                 for (int r = 0; r < 4; r++) worst[r] = u16x2{0, 0};
-                if (c == 0 || c == nchunks - 1) {            // places before the partition's first point or past its last
+                if (c == 0 || c == nchunks - 1) {            // places before the run's first or past its last
 #pragma unroll
                     for (int r = 0; r < 4; r++) {
-                        const bool out0 = (uint32_t)(first + 2 * r) >= (uint32_t)n;
-                        const bool out1 = (uint32_t)(first + 2 * r + 1) >= (uint32_t)n;
+                        const bool out0 = first + 2 * r < run_lo || first + 2 * r >= run_hi;
+                        const bool out1 = first + 2 * r + 1 < run_lo || first + 2 * r + 1 >= run_hi;
                         worst[r] = u16x2{(uint16_t)(out0 ? 0xffff : 0), (uint16_t)(out1 ? 0xffff : 0)};
                     }
                 }
-                const uint16_t* at = inv_m + 8 * (int64_t)c;
+                // (a row's start is the same for every thread and the chunk's offset a 32-bit number:
+                //  scalar base + vector offset addressing, no 64-bit address per thread and row)
+                const uint32_t chunk_bytes = (uint32_t)c * 16u;
                 auto group = [&](int h0, auto width) {
                     constexpr int W = decltype(width)::value;
                     u32x4 x[W];
 #pragma unroll
-                    for (int u = 0; u < W; u++) x[u] = *(g_u32x4*)(at + (int64_t)(h0 + u) * a.N);
+                    for (int u = 0; u < W; u++) {
+                        const char* row = reinterpret_cast<const char*>(rp + (int64_t)(h0 + u) * a.N);
+                        x[u] = *(g_u32x4*)(row + chunk_bytes);
+                    }
 #pragma unroll
                     for (int u = 0; u < W; u++) {
                         const u16x2 lo = __builtin_bit_cast(u16x2, lo2[h0 + u]);
@@ -373,7 +387,7 @@ __global__ __launch_bounds__(NT, MINW) void traverse_block_kernel(QueryArgs a, B
                         }
                     }
                 };
-                int h0 = 0;
+                int h0 = 1;
                 for (; h0 + 4 <= a.L; h0 += 4) group(h0, std::integral_constant<int, 4>());
                 if (h0 + 2 <= a.L) { group(h0, std::integral_constant<int, 2>()); h0 += 2; }
                 if (h0 < a.L) group(h0, std::integral_constant<int, 1>());
@@ -385,13 +399,15 @@ __global__ __launch_bounds__(NT, MINW) void traverse_block_kernel(QueryArgs a, B
                 for (int e = 0; e < 8; e++) {
                     const uint32_t w = __builtin_bit_cast(uint32_t, worst[e >> 1]);
                     if (((w >> ((e & 1) * 16)) & 0xffffu) != 0u) continue;
-                    const uint32_t local = (uint32_t)(first + e);
+                    // the point standing at that place of the first index's slice
+                    const uint32_t local = (uint32_t)(a.sids[first_row + first + e] - (int32_t)off);
                     if ((marked_m[local >> 5] >> (local & 31u)) & 1u) continue;
                     const uint32_t slot = atomicAdd(&misc[kPromoCount], 1u);
                     if (slot < (uint32_t)y.promo_cap) promo[slot] = local | ((uint32_t)m << 26);
                 }
             }
         }
+        return looked_at;
     };
     auto mark_promotions = [&](uint32_t np) {
         for (uint32_t j = tid; j < np; j += NT) {
@@ -474,8 +490,13 @@ __global__ __launch_bounds__(NT, MINW) void traverse_block_kernel(QueryArgs a, B
         PHASE_END(2);
 
         // ---- 3. the points whose L windows are now all consumed ---------------------
-        scan_epoch();
-        if (a.counters && tid == 0) atomicAdd(&misc[kScannedLo], 1u);      // scans so far, each over n * I index entries
+        {
+            const unsigned long long looked_at = scan_epoch();
+            if (a.counters && tid == 0) {       // (a 64-bit count in two words of the workgroup's scalars)
+                const unsigned long long sum = (((unsigned long long)misc[kScannedHi] << 32) | misc[kScannedLo]) + looked_at;
+                misc[kScannedLo] = (uint32_t)sum; misc[kScannedHi] = (uint32_t)(sum >> 32);
+            }
+        }
         __syncthreads();
         PHASE_END(3);
         const uint32_t np = misc[kPromoCount];
@@ -910,7 +931,7 @@ __global__ __launch_bounds__(NT, MINW) void traverse_block_kernel(QueryArgs a, B
             } else {
                 steps = min(bound, maxw + 1);
             }
-            const unsigned long long st = (unsigned long long)misc[kScannedLo] * (unsigned long long)n * (unsigned long long)I;
+            const unsigned long long st = ((unsigned long long)misc[kScannedHi] << 32) | misc[kScannedLo];
             atomicAdd(&a.counters[(int64_t)qi * 4 + 0], st);
             atomicAdd(&a.counters[(int64_t)qi * 4 + 1], (unsigned long long)misc[kNumCand]);
             atomicAdd(&a.counters[(int64_t)qi * 4 + 2], (unsigned long long)misc[kProbes]);
@@ -930,7 +951,7 @@ bool block_traversal_supported(const QueryArgs& a, size_t* lds_bytes) {
     const BlockLayout y = make_block_layout(a);
     if (lds_bytes) *lds_bytes = y.lds_bytes;
     const int I = a.M * a.L;
-    if (!a.inv || a.ppb > 65536) return false;             // positions inside a slice are 16-bit values
+    if (!a.inv || !a.rpos || !a.rpos_ready || a.ppb > 65536) return false;   // positions inside a slice are 16-bit values
     if (4 * I > kBlockThreads || a.M > 64) return false;   // lane groups per stream in the searches; composite number in 6 bits
     if (a.kcap > 512) return false;
     if (a.ppb >= (1 << 25)) return false;

@@ -32,7 +32,8 @@ enum {
 
 /* Per-query traversal counters written by dcih_query when asked for. */
 enum {
-    DCIH_CTR_VISITED = 0,   /* in-range index entries visited            */
+    DCIH_CTR_VISITED = 0,   /* in-range index entries visited (step-by-step kernel: the reference loop's
+                               count exactly; the other kernels: the index entries they read)  */
     DCIH_CTR_CANDIDATES = 1,/* points promoted = exact distances computed */
     DCIH_CTR_PROBES = 2,    /* key reads made by the positioning search   */
     DCIH_CTR_STEPS = 3,     /* outer steps executed, summed over partitions */

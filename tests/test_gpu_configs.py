@@ -55,8 +55,6 @@ def _l1(gpu, oracle, dci, X, Q, M, L, B, T, k, outer, modes):
         ids, dists, ctr = ids.cpu().numpy(), dists.cpu().numpy(), ctr.cpu().numpy()
         if mode == "step":
             np.testing.assert_array_equal(ctr[:, 0], rc[:, 0], err_msg="entries visited (%s)" % mode)
-        else:
-            assert np.all(ctr[:, 0] >= rc[:, 0]), mode
         np.testing.assert_array_equal(ctr[:, 1], rc[:, 1], err_msg="candidates promoted (%s)" % mode)
         np.testing.assert_array_equal(ctr[:, 3], rc[:, 3], err_msg="outer steps (%s)" % mode)
         np.testing.assert_allclose(dists, ref["dists"], rtol=DIST_RTOL, atol=1e-6)

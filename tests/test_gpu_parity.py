@@ -60,8 +60,7 @@ def _assert_l1(ids, dists, ctr, ref, exact_ids=True, visits=True):
     rc = ref["counters"].astype(np.int64)
     if visits:
         np.testing.assert_array_equal(ctr[:, 0], rc[:, 0], err_msg="entries visited")
-    else:   # the batch kernel streams whole epochs: never fewer entries than the loop visits
-        assert np.all(ctr[:, 0] >= rc[:, 0])
+    # (the other kernels count the index entries they read, which the loop's visits do not bound)
     np.testing.assert_array_equal(ctr[:, 1], rc[:, 1], err_msg="candidates promoted")
     np.testing.assert_array_equal(ctr[:, 3], rc[:, 3], err_msg="outer steps")
     np.testing.assert_allclose(dists, ref["dists"], rtol=DIST_RTOL, atol=1e-6)
