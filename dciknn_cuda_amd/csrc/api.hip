@@ -544,6 +544,7 @@ static int query_impl(dcih_index* h, int dim, int num_queries, const float* d_qu
     QueryArgs a;
     a.skeys = h->d_skeys; a.sids = h->d_sids; a.inv = h->d_inv; a.data = h->d_data; a.query = d_query;
     a.rpos = h->d_rpos; a.rpos_ready = &h->rpos_ready;
+    a.hints_cold = 0;
     a.mode = h->traversal; a.item_list = nullptr; a.item_count = nullptr; a.dense = nullptr;
     a.xcds = h->xcds; a.q_first = 0; a.q_count = num_queries;
     a.dense_items = nullptr; a.dense_count = nullptr; a.dense_cap = 0;
@@ -557,6 +558,7 @@ static int query_impl(dcih_index* h, int dim, int num_queries, const float* d_qu
         if (rc) return rc;
         h->hint_k = num_neighbours; h->hint_outer = num_outer_iterations;
         h->hint_T = thread_size; h->hint_maxc = max_num_candidates;
+        a.hints_cold = 1;
     }
     a.stop_hint = h->d_stop_hint;
     a.N = h->n;

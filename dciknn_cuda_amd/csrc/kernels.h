@@ -71,6 +71,7 @@ struct QueryArgs {
     const int32_t* item_list;    // step-by-step kernel: null = all nq*B items, else this list
     const uint32_t* item_count;  // ... of this length
     float* stop_hint;        // null, or [3][B] per partition: running averages of the stop step and of the promotions at the stop, stops seen
+    int hints_cold;          // the table was cleared for this call: nothing is known yet about where traversals stop
     unsigned long long* phase_ticks;  // null, or 16 accumulators for the batch kernel's phases
     int mode;                // 0 = pick, 1 = step-by-step kernel, 2 = batch kernel, 3 = dense kernel
     // hand-over from the batch kernel to the dense kernel: one list of items per die

@@ -907,7 +907,7 @@ __global__ __launch_bounds__(NT, MINW) void traverse_block_kernel(QueryArgs a, B
         atomicAdd(&a.phase_ticks[9], 1ull);
     }
     if (a.stop_hint && tid == 0 && misc[kStop])
-        record_stop(a.stop_hint, a.B, b, (float)((((unsigned long long)misc[kStopStepHi] << 32) | misc[kStopStepLo]) + 1),
+        record_stop(a.stop_hint, a.B, b, qi, (float)((((unsigned long long)misc[kStopStepHi] << 32) | misc[kStopStepLo]) + 1),
                     (float)(misc[kNumCand] + misc[kEventCount]));
     // ---- results -------------------------------------------------------------------
     const int topn = (int)misc[kTopN];
@@ -941,6 +941,7 @@ __global__ __launch_bounds__(NT, MINW) void traverse_block_kernel(QueryArgs a, B
 }
 
 constexpr int kBlockThreads = 256;
+constexpr int kLeadQueries = 32;
 
 #undef PHASE_END
 #undef PHASE_FENCE
@@ -967,10 +968,15 @@ int query_block(const QueryArgs& a_in, hipStream_t s) {
     // as many queries per launch as the launch limit allows (nearly always all of them)
     const int per_launch = block_queries_per_launch(a_in.xcds, a_in.B, a_in.nq);
     if (per_launch < 1) return fail(-4, "query: block_size too large for the batch traversal kernel");
-    for (int q0 = 0; q0 < a_in.nq; q0 += per_launch) {
+    // With nothing known yet about where traversals stop, a few queries go ahead in a launch of
+    // their own: their stops are on record when the others start, which then size their first
+    // epoch from them instead of feeling their way forward (the first resident round of every
+    // partition would otherwise do that in the middle of the large launch).  Results do not depend on it.
+    const int lead = a_in.hints_cold && a_in.stop_hint && a_in.nq >= 8 * kLeadQueries ? kLeadQueries : 0;
+    for (int q0 = 0; q0 < a_in.nq; q0 += (q0 < lead ? lead : per_launch)) {
         QueryArgs a = a_in;
         a.q_first = q0;
-        a.q_count = min(per_launch, a_in.nq - q0);
+        a.q_count = q0 < lead ? lead : min(per_launch, a_in.nq - q0);
         const int64_t items = block_items(a.xcds, a.B, a.q_count);
 #define DCIH_LAUNCH(MW)                                                                            \
     do {                                                                                           \

@@ -101,9 +101,15 @@ __device__ inline int group_partition_point(int lo, int hi, bool active, int lg,
 // partition.  Many workgroups record at once, so the sums are formed by atomic additions; a
 // partition stops recording after kHintStops stops, which makes the averages (and with them
 // the sizes of the batch kernel's epochs) the same from then on.  They steer work, never results.
-constexpr float kHintStops = 4096.0f;
-__device__ inline void record_stop(float* stop_hint, int B, int b, float steps, float promotions) {
-    if (stop_hint[2 * B + b] >= kHintStops) return;
+// All workgroups an accelerator die runs at one time work on the same partition, so their additions
+// hit the same three words and queue up behind each other (a quarter more time for a whole call
+// when every stop is recorded): after the first kHintEveryStop stops only every eighth query's
+// stops are recorded, which spreads the same number of samples over eight times as many stops.
+constexpr float kHintStops = 512.0f;
+constexpr float kHintEveryStop = 64.0f;
+__device__ inline void record_stop(float* stop_hint, int B, int b, int query, float steps, float promotions) {
+    const float have = stop_hint[2 * B + b];
+    if (have >= kHintStops || (have >= kHintEveryStop && (query & 7) != 0)) return;
     atomicAdd(&stop_hint[b], steps);
     atomicAdd(&stop_hint[B + b], promotions);
     atomicAdd(&stop_hint[2 * B + b], 1.0f);

@@ -814,7 +814,7 @@ __global__ __launch_bounds__(kDT, WPS) void traverse_dense_kernel(QueryArgs a, D
         const unsigned long long bound = (unsigned long long)n * a.L * T;
         unsigned long long steps = min(bound, maxw + 1);
         if (stop) steps = min(t_stop + 1, steps);
-        if (a.stop_hint && tid == 0 && stop) record_stop(a.stop_hint, a.B, b, (float)(t_stop + 1), (float)misc[dCand]);
+        if (a.stop_hint && tid == 0 && stop) record_stop(a.stop_hint, a.B, b, qi, (float)(t_stop + 1), (float)misc[dCand]);
         if (a.counters) {
             for (int o = 32; o > 0; o >>= 1) probes += (uint32_t)__shfl_xor((int)probes, o, kWave);
             if (lane == 0) atomicAdd(&misc[dProbes], probes);
