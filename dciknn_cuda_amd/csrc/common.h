@@ -86,6 +86,18 @@ template <int O> __device__ inline unsigned long long lane_xor(unsigned long lon
     return ((unsigned long long)lane_xor_u32<O>((uint32_t)(v >> 32)) << 32) | lane_xor_u32<O>((uint32_t)v);
 }
 
+// The same for a distance that is a constant only after loop unrolling.
+__device__ inline unsigned long long lane_xor_any(unsigned long long v, int o) {
+    switch (o) {
+        case 1: return lane_xor<1>(v);
+        case 2: return lane_xor<2>(v);
+        case 4: return lane_xor<4>(v);
+        case 8: return lane_xor<8>(v);
+        case 16: return lane_xor<16>(v);
+        default: return lane_xor<32>(v);
+    }
+}
+
 // ---- wavefront (64-lane) reductions ----------------------------------------
 // (levels in the order 32, 16, .., 1: the traversal kernels rely on this order for equal bits)
 __device__ inline float wave_sum(float v) {
@@ -284,7 +296,7 @@ __device__ inline void bitonic_sort_u64_regs(unsigned long long* s) {
 #pragma unroll
                 for (int i = 0; i < E; i++) {
                     const int e = tid * E + i;
-                    const unsigned long long o = __shfl_xor(v[i], stride / E, kWave);
+                    const unsigned long long o = lane_xor_any(v[i], stride / E);
                     const bool keep_min = ((e & stride) == 0) == ((e & size) == 0);
                     v[i] = keep_min ? (v[i] < o ? v[i] : o) : (v[i] > o ? v[i] : o);
                 }

@@ -112,7 +112,7 @@ __device__ inline float group_row_sums(float (&v)[N], int s) {
         for (int i = 0; i < H; i++) {
             const float send = upper ? v[i] : v[i + H];
             const float keep = upper ? v[i + H] : v[i];
-            nv[i] = keep + __shfl_xor(send, H, kWave);
+            nv[i] = keep + lane_xor<H>(send);
         }
         return group_row_sums<H>(nv, s);
     }
@@ -816,7 +816,7 @@ __global__ __launch_bounds__(kDT, WPS) void traverse_dense_kernel(QueryArgs a, D
         if (stop) steps = min(t_stop + 1, steps);
         if (a.stop_hint && tid == 0 && stop) record_stop(a.stop_hint, a.B, b, qi, (float)(t_stop + 1), (float)misc[dCand]);
         if (a.counters) {
-            for (int o = 32; o > 0; o >>= 1) probes += (uint32_t)__shfl_xor((int)probes, o, kWave);
+            probes = wave_sum_u32(probes);
             if (lane == 0) atomicAdd(&misc[dProbes], probes);
             __syncthreads();
             if (tid == 0) {
