@@ -990,9 +990,10 @@ int query_block(const QueryArgs& a_in, hipStream_t s) {
         hipLaunchKernelGGL((traverse_block_kernel<kBlockThreads, MW>), dim3((unsigned)items),      \
                            dim3(kBlockThreads), y.lds_bytes, s, a, y);                             \
     } while (0)
-        // (measured on 1M x 128, 17858-point partitions: 5 -> 223 k, 6 -> 235 k, 7 and 8 -> 241 k queries/s)
+        // (measured on 1M x 128, 17858-point partitions: 5 -> 275 k, 6 -> 301 k, 7 -> 309 k, 8 -> 287 k queries/s:
+        //  eight workgroups per CU leave 64 registers, which spill; that variant is not built)
         int minw = fit >= 7 ? 7 : (fit < 3 ? 3 : fit);
-        if (minw >= 8) DCIH_LAUNCH(8); else if (minw == 7) DCIH_LAUNCH(7); else if (minw == 6) DCIH_LAUNCH(6);
+        if (minw >= 7) DCIH_LAUNCH(7); else if (minw == 6) DCIH_LAUNCH(6);
         else if (minw == 5) DCIH_LAUNCH(5); else if (minw == 4) DCIH_LAUNCH(4); else DCIH_LAUNCH(3);
 #undef DCIH_LAUNCH
         DCIH_HIP(hipGetLastError());
