@@ -46,6 +46,7 @@ SIGNATURES = {
     "dcih_get_index": (_c.c_int, [_c.c_void_p, _c.c_void_p, _c.c_void_p]),
     "dcih_set_option": (_c.c_int, [_c.c_void_p, _c.c_int, _c.c_int]),
     "dcih_phase_profile": (_c.c_int, [_c.c_void_p, _c.c_void_p]),
+    "dcih_debug_positions": (_c.c_int, [_c.c_void_p, _c.c_void_p, _c.c_void_p, _c.c_void_p]),
     "dcih_profile": (_c.c_int, [_c.c_void_p, _c.c_int]),
     "dcih_last_timings": (_c.c_int, [_c.c_void_p, _c.c_void_p]),
     "dcih_num_points": (_c.c_int64, [_c.c_void_p]),

@@ -697,6 +697,28 @@ int64_t dcih_debug_launch_map(int xcds, int block_size, int num_queries, int64_t
     return items;
 }
 
+int dcih_debug_positions(dcih_index* h, uint16_t* d_inv, uint16_t* d_rpos, void* stream) {
+    if (!h) return fail(DCIH_EINVAL, "dcih_debug_positions: null handle");
+    if (h->n <= 0) return fail(DCIH_ESTATE, "dcih_debug_positions: the index is empty");
+    if (!h->d_inv || !h->d_rpos) return fail(DCIH_EUNSUPPORTED, "dcih_debug_positions: this index keeps no position tables");
+    DeviceGuard guard(h->device);
+    hipStream_t s = (hipStream_t)stream;
+    const size_t cells = (size_t)num_indices(h) * (size_t)h->n;
+    if (d_inv) DCIH_HIP(hipMemcpyAsync(d_inv, h->d_inv, cells * sizeof(uint16_t), hipMemcpyDeviceToDevice, s));
+    if (d_rpos) {
+        if (!h->rpos_ready) {
+            // (rows of the first simple indices are never written: clear the table so that they read as zeros)
+            DCIH_HIP(hipMemsetAsync(h->d_rpos, 0, cells * sizeof(uint16_t), s));
+            const int rc = fill_positions_by_first(h->d_sids, h->d_inv, h->d_rpos, h->n, h->M, h->L, s);
+            if (rc) return rc;
+            h->rpos_ready = 1;
+        }
+        DCIH_HIP(hipMemcpyAsync(d_rpos, h->d_rpos, cells * sizeof(uint16_t), hipMemcpyDeviceToDevice, s));
+    }
+    DCIH_HIP(hipStreamSynchronize(s));
+    return DCIH_OK;
+}
+
 int dcih_set_option(dcih_index* h, int option, int value) {
     if (!h) return fail(DCIH_EINVAL, "dcih_set_option: null handle");
     if (option == DCIH_OPT_TRAVERSAL && value >= 0 && value <= 3) {

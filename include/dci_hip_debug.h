@@ -34,6 +34,18 @@ int dcih_phase_profile(dcih_index* h, uint64_t* d_ticks);
 int64_t dcih_debug_launch_map(int xcds, int block_size, int num_queries, int64_t block,
                               int* b, int* q, int* queries_per_launch);
 
+/*
+ * The two position tables of the index (no counterpart in the reference, which keeps only
+ * (key, id) pairs): d_inv and d_rpos each receive [num_indices][num_points] uint16 values, or
+ * may be NULL.  inv[i][p] = place of point p in the sorted slice of simple index i that holds
+ * it; rpos[i][e] = inv[i][id at element e of the FIRST simple index of i's composite], i.e.
+ * the same places in that index's order (the rows of the first simple indices themselves are
+ * never written and come back as zeros).  The second table is filled here if no query has
+ * needed it yet.  DCIH_EUNSUPPORTED for an index whose partitions exceed 65536 points (it
+ * keeps neither table).  Synchronises the stream.
+ */
+int dcih_debug_positions(dcih_index* h, uint16_t* d_inv, uint16_t* d_rpos, void* stream);
+
 #ifdef __cplusplus
 }
 #endif

@@ -146,6 +146,42 @@ def test_index_arrays_are_consistent(gpu):
         dci.free()
 
 
+@pytest.mark.parametrize("fill_by", ["accessor", "query"])
+def test_position_tables(gpu, fill_by):
+    """inv is the inverse of every sorted slice; rpos holds the same places in the order of the first
+    simple index of each composite (the table the batch traversal scans), whether the inspection call
+    or the first batch traversal fills it."""
+    from dciknn_cuda_amd import _capi
+    rng = np.random.default_rng(11)
+    for n, B, M, L in [(40_000, 2, 2, 3), (9_001, 3, 3, 4), (1_000, 5, 1, 2), (777, 4, 2, 1), (4_096, 1, 2, 5)]:
+        X = rng.standard_normal((n, 8)).astype(np.float32)
+        dci = gpu.DCI(8, M, L, B, 4, seed=3, traversal="batch")
+        dci.add(torch.from_numpy(X).cuda())
+        if fill_by == "query":
+            dci.query(torch.from_numpy(X[:5]).cuda(), 3, 20)
+        I = M * L
+        d_inv = torch.zeros((I, n), dtype=torch.int16, device="cuda")
+        d_rpos = torch.zeros((I, n), dtype=torch.int16, device="cuda")
+        _capi.check(dci._lib.dcih_debug_positions(dci._dci_inst, d_inv.data_ptr(), d_rpos.data_ptr(), None))
+        inv = d_inv.cpu().numpy().view(np.uint16).astype(np.int64)
+        rpos = d_rpos.cpu().numpy().view(np.uint16).astype(np.int64)
+        _, si = engine_index(dci)
+        ppb = -(-n // B)
+        for b in range(B):
+            lo, hi = b * ppb, min(n, (b + 1) * ppb)
+            if hi <= lo:
+                continue
+            places = np.arange(hi - lo)
+            for i in range(I):
+                ids = si[i, lo:hi]
+                np.testing.assert_array_equal(inv[i, ids], places, err_msg="inv, index %d partition %d" % (i, b))
+                first = (i // L) * L
+                if i != first:      # (the first indices' own rows are never written)
+                    np.testing.assert_array_equal(rpos[i, lo:hi], inv[i, si[first, lo:hi]],
+                                                  err_msg="rpos, index %d partition %d" % (i, b))
+        dci.free()
+
+
 def test_segsort_invariants_large(gpu):
     """Size-independent properties at a partition length beyond one LDS tile."""
     n, I, B = 300_000, 2, 2
