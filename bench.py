@@ -68,7 +68,7 @@ OTHER_LEGS = [
 # soon as 50 windows' first points are promoted).
 TUNED = {
     "c1": dict(bs=100, ts=10, outer=5000),
-    "c2": dict(bs=56, ts=2, outer=500),
+    "c2": dict(bs=58, ts=2, outer=500),
     "c3": dict(bs=400, ts=128, outer=100),
     "c4": dict(bs=100, ts=64, outer=126),
     "c5": dict(bs=900, ts=128, outer=10),

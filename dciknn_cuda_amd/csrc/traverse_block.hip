@@ -82,7 +82,7 @@ BlockLayout make_block_layout(const QueryArgs& a) {
     // is redone by the step-by-step kernel
     // The tables grow with the promotions a stop needs (about k * T, more when the
     // step limit rather than c0 >= k ends the traversal): fewer, larger epochs.
-    y.promo_cap = 256;
+    y.promo_cap = 128;
     while (y.promo_cap < 2 * (int64_t)a.k_stop * a.T && y.promo_cap < 2048) y.promo_cap <<= 1;
     y.promo_max = y.promo_cap * 5 / 8;
     y.event_cap = 2 * y.promo_cap;
@@ -941,6 +941,7 @@ __global__ __launch_bounds__(NT, MINW) void traverse_block_kernel(QueryArgs a, B
 }
 
 constexpr int kBlockThreads = 256;
+constexpr int kNarrowThreads = 128;     // workgroups of two wavefronts: more (query, partition) items per CU
 constexpr int kLeadQueries = 32;
 
 #undef PHASE_END
@@ -978,23 +979,38 @@ int query_block(const QueryArgs& a_in, hipStream_t s) {
         a.q_first = q0;
         a.q_count = q0 < lead ? lead : min(per_launch, a_in.nq - q0);
         const int64_t items = block_items(a.xcds, a.B, a.q_count);
-#define DCIH_LAUNCH(MW)                                                                            \
+#define DCIH_LAUNCH(NT, MW)                                                                        \
     do {                                                                                           \
         static DeviceOnce once;                                                                    \
         const int rc_attr = once.run([]() -> int {                                                 \
-            DCIH_HIP(hipFuncSetAttribute((const void*)traverse_block_kernel<kBlockThreads, MW>,    \
+            DCIH_HIP(hipFuncSetAttribute((const void*)traverse_block_kernel<NT, MW>,               \
                                          hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024)); \
             return 0;                                                                              \
         });                                                                                        \
         if (rc_attr) return rc_attr;                                                               \
-        hipLaunchKernelGGL((traverse_block_kernel<kBlockThreads, MW>), dim3((unsigned)items),      \
-                           dim3(kBlockThreads), y.lds_bytes, s, a, y);                             \
+        hipLaunchKernelGGL((traverse_block_kernel<NT, MW>), dim3((unsigned)items),                 \
+                           dim3(NT), y.lds_bytes, s, a, y);                                        \
     } while (0)
-        // (measured on 1M x 128, 17858-point partitions: 5 -> 275 k, 6 -> 301 k, 7 -> 309 k, 8 -> 287 k queries/s:
-        //  eight workgroups per CU leave 64 registers, which spill; that variant is not built)
-        int minw = fit >= 7 ? 7 : (fit < 3 ? 3 : fit);
-        if (minw >= 7) DCIH_LAUNCH(7); else if (minw == 6) DCIH_LAUNCH(6);
-        else if (minw == 5) DCIH_LAUNCH(5); else if (minw == 4) DCIH_LAUNCH(4); else DCIH_LAUNCH(3);
+        // The kernel's time is chains of dependent reads, so what counts is how many items a CU holds: as
+        // many as LDS lets in, with the registers that leaves (wavefronts per SIMD = the second template
+        // argument).  Where few promotions are expected and LDS lets ten or more items in, the workgroup
+        // is two wavefronts instead of four: half the threads per item, more items within the same
+        // registers (1M x 128, 17858-point partitions, four wavefronts: 5 / 6 / 7 / 8 workgroups per CU
+        // 275 / 301 / 309 / 287 k queries/s, eight spilling; two wavefronts, ten workgroups: 326 k; with
+        // nine or fewer items per CU -- partitions above ~22 k points -- two wavefronts lose: 287 against
+        // 300 k at 26316 points, 224 against 279 k at 35715).
+        const bool narrow = 4 * a.M * a.L <= kNarrowThreads && y.promo_cap <= 128 && fit >= 10;
+        int minw = narrow ? (fit * (kNarrowThreads / 64) + 3) / 4 : fit;      // wavefronts per SIMD
+        minw = minw >= 7 ? 7 : (minw < 3 ? 3 : minw);
+        if (narrow) {
+            if (minw >= 7) DCIH_LAUNCH(kNarrowThreads, 7); else if (minw == 6) DCIH_LAUNCH(kNarrowThreads, 6);
+            else if (minw == 5) DCIH_LAUNCH(kNarrowThreads, 5); else if (minw == 4) DCIH_LAUNCH(kNarrowThreads, 4);
+            else DCIH_LAUNCH(kNarrowThreads, 3);
+        } else {
+            if (minw >= 7) DCIH_LAUNCH(kBlockThreads, 7); else if (minw == 6) DCIH_LAUNCH(kBlockThreads, 6);
+            else if (minw == 5) DCIH_LAUNCH(kBlockThreads, 5); else if (minw == 4) DCIH_LAUNCH(kBlockThreads, 4);
+            else DCIH_LAUNCH(kBlockThreads, 3);
+        }
 #undef DCIH_LAUNCH
         DCIH_HIP(hipGetLastError());
     }
