@@ -33,6 +33,7 @@
 // many points at once is dropped and retried smaller.  Whatever does not fit the
 // fixed LDS tables is handed to the step-by-step kernel through a redo list, so
 // results never depend on which kernel produced them.
+#include <cmath>
 #include <type_traits>
 
 #include "common.h"
@@ -82,8 +83,15 @@ BlockLayout make_block_layout(const QueryArgs& a) {
     // is redone by the step-by-step kernel
     // The tables grow with the promotions a stop needs (about k * T, more when the
     // step limit rather than c0 >= k ends the traversal): fewer, larger epochs.
+    // (the step limit can ask for more than k * T: a traversal that must consume the fraction f of a
+    //  composite's windows before it may stop has by then promoted about f^L of the partition, unless
+    //  max_candidates first-lane promotions end it earlier -- the estimate the kernel choice uses)
+    const double windows = (double)a.L * ((double)a.ppb / (double)a.T);
+    const double f = fmin(1.0, (double)a.stop_at / fmax(1.0, windows));
+    const double by_steps = fmin((double)a.ppb * pow(f, (double)a.L), (double)a.max_cand * (double)a.T);
+    const double expected = fmax((double)a.k_stop * (double)a.T, by_steps);
     y.promo_cap = 128;
-    while (y.promo_cap < 2 * (int64_t)a.k_stop * a.T && y.promo_cap < 2048) y.promo_cap <<= 1;
+    while ((double)y.promo_cap < 2.0 * expected && y.promo_cap < 2048) y.promo_cap <<= 1;
     y.promo_max = y.promo_cap * 5 / 8;
     y.event_cap = 2 * y.promo_cap;
     y.sort_cap = 64;           // top-k plus a batch of at least 48 new candidates
