@@ -59,7 +59,6 @@ struct BlockLayout {
     int off_idx;      // per simple index: p, qp, and the visited run as packed 16-bit pairs (4 * I words)
     int off_stream;   // per stream: consumed, previous, total, stride, composite number (5 * 2I words)
     int off_comp;     // per composite: rho bits, K, active, previous K, sum of inverse priorities, scan flag (6 * M words)
-    int off_q;        // query row
     int off_samp;     // per stream: 16 sampled window priorities of the current epoch's range
     int off_promo, off_events, off_acc, off_sort, off_flags;
     int promo_cap;    // promotions one epoch may produce (table size)
@@ -78,7 +77,6 @@ BlockLayout make_block_layout(const QueryArgs& a) {
     y.off_idx = o;      o += 4 * I * 4;
     y.off_stream = o;   o += 5 * 2 * I * 4;
     y.off_comp = o;     o += 6 * a.M * 4;
-    y.off_q = o;        o += ((a.dim + 3) & ~3) * 4;
     // small tables keep more workgroups resident per CU; an item that overflows them
     // is redone by the step-by-step kernel
     // The tables grow with the promotions a stop needs (about k * T, more when the
@@ -132,7 +130,6 @@ __global__ __launch_bounds__(NT, MINW) void traverse_block_kernel(QueryArgs a, B
     uint32_t* s_Kprev = s_active + a.M;
     float* s_hsum = reinterpret_cast<float*>(s_Kprev + a.M);
     uint32_t* s_noscan = reinterpret_cast<uint32_t*>(s_hsum + a.M);   // some simple index of the composite has visited nothing yet
-    float* s_q = reinterpret_cast<float*>(smem + y.off_q);
     uint32_t* s_samp = reinterpret_cast<uint32_t*>(smem + y.off_samp);
     uint32_t* promo = reinterpret_cast<uint32_t*>(smem + y.off_promo);
     uint32_t* acc = reinterpret_cast<uint32_t*>(smem + y.off_acc);
@@ -240,7 +237,6 @@ __global__ __launch_bounds__(NT, MINW) void traverse_block_kernel(QueryArgs a, B
 
     // ---- set-up ---------------------------------------------------------------
     for (int w = tid; w < y.flag_words; w += NT) seen[w] = 0;
-    for (int j = tid; j < a.dim; j += NT) s_q[j] = a.query[(int64_t)qi * a.dim + j];
     uint32_t probes = 0;
     {   // positioning search (:279-297): first position whose key is not below qp,
         // one group of lanes per simple index
@@ -827,7 +823,9 @@ __global__ __launch_bounds__(NT, MINW) void traverse_block_kernel(QueryArgs a, B
                 const int64_t pt1 = c2 < batch ? off + acc[done + c2] : pt0;
                 const float* const rows2[2] = {a.data + pt0 * a.dim, a.data + pt1 * a.dim};
                 float d2[2];
-                wave_row_dists<2>(rows2, s_q, a.dim, vec4, d2, lane);
+                // (the query's row comes from global memory: it is read a few dozen times per item, and the
+                //  room it took in LDS decides at some settings whether one more item fits a CU)
+                wave_row_dists<2>(rows2, a.query + (int64_t)qi * a.dim, a.dim, vec4, d2, lane);
                 if (lane == 0) {
                     sortbuf[topn + c] = ((unsigned long long)__builtin_bit_cast(uint32_t, d2[0]) << 32) | (uint32_t)pt0;
                     if (c2 < batch)
