@@ -45,6 +45,8 @@ namespace dcih {
 namespace {
 
 constexpr int kMaxEpochs = 100000;
+constexpr int kSampleShift = 3;       // 2^shift - 1 window priorities sampled per stream and epoch
+constexpr int kSamples = 1 << kSampleShift;
 
 
 enum Misc {   // 32-bit scalars shared by the workgroup
@@ -59,7 +61,7 @@ struct BlockLayout {
     int off_idx;      // per simple index: p, qp, and the visited run as packed 16-bit pairs (4 * I words)
     int off_stream;   // per stream: consumed, previous, total, stride, composite number (5 * 2I words)
     int off_comp;     // per composite: rho bits, K, active, previous K, sum of inverse priorities, scan flag (6 * M words)
-    int off_samp;     // per stream: 16 sampled window priorities of the current epoch's range
+    int off_samp;     // per stream: kSamples - 1 sampled window priorities of the current epoch's range (slot 0 unused)
     int off_promo, off_events, off_acc, off_sort, off_flags;
     int promo_cap;    // promotions one epoch may produce (table size)
     int promo_max;    // above this an epoch is dropped and halved
@@ -99,8 +101,8 @@ BlockLayout make_block_layout(const QueryArgs& a) {
     y.off_samp = o;
     y.off_acc = o;
     // (blind querying keeps the promoting step beside every accepted candidate)
-    o += max(2 * I * 16 * 4 + y.promo_cap * 4, y.event_cap * 4 * (a.blind ? 2 : 1));
-    y.off_promo = y.off_samp + 2 * I * 16 * 4;
+    o += max(2 * I * kSamples * 4 + y.promo_cap * 4, y.event_cap * 4 * (a.blind ? 2 : 1));
+    y.off_promo = y.off_samp + 2 * I * kSamples * 4;
     o = (o + 15) & ~15;
     y.off_events = o;   o += y.event_cap * 8;
     y.off_sort = o;     o += y.sort_cap * 8;
@@ -392,8 +394,7 @@ __global__ __launch_bounds__(NT, MINW) void traverse_block_kernel(QueryArgs a, B
                     }
                 };
                 int h0 = 1;
-                for (; h0 + 4 <= a.L; h0 += 4) group(h0, std::integral_constant<int, 4>());
-                if (h0 + 2 <= a.L) { group(h0, std::integral_constant<int, 2>()); h0 += 2; }
+                for (; h0 + 2 <= a.L; h0 += 2) group(h0, std::integral_constant<int, 2>());
                 if (h0 < a.L) group(h0, std::integral_constant<int, 1>());
                 const u16x2 m01 = __builtin_elementwise_min(worst[0], worst[1]);
                 const u16x2 m23 = __builtin_elementwise_min(worst[2], worst[3]);
@@ -531,12 +532,12 @@ __global__ __launch_bounds__(NT, MINW) void traverse_block_kernel(QueryArgs a, B
 
         // ---- 4. exact step of every promotion -----------------------------------
         if (np > 0) {     // sample every stream's new range once; all rankings of the epoch share it
-            for (int idx = tid; idx < S * 15; idx += NT) {
-                const int sidx = idx / 15, t = idx - sidx * 15 + 1;
+            for (int idx = tid; idx < S * (kSamples - 1); idx += NT) {
+                const int sidx = idx / (kSamples - 1), t = idx - sidx * (kSamples - 1) + 1;
                 const int lo = s_cprev[sidx], len = s_c[sidx] - lo;
                 if (len >= 32) {
                     probes++;
-                    s_samp[sidx * 16 + t] = stream_prio_bits(load_stream(sidx), lo + (int)(((uint32_t)len * (uint32_t)t) >> 4));
+                    s_samp[sidx * kSamples + t] = stream_prio_bits(load_stream(sidx), lo + (int)(((uint32_t)len * (uint32_t)t) >> kSampleShift));
                 }
             }
             __syncthreads();
@@ -618,16 +619,16 @@ __global__ __launch_bounds__(NT, MINW) void traverse_block_kernel(QueryArgs a, B
                         if (len >= 32) {
                             // the samples ascend: the number of them ordered before the window
                             // is the last such sample's index (independent reads, no search)
-                            const uint32_t* tab = s_samp + sidx * 16;
+                            const uint32_t* tab = s_samp + sidx * kSamples;
                             int tl = 0;
 #pragma unroll
-                            for (int t2 = 1; t2 < 16; t2++) {
+                            for (int t2 = 1; t2 < kSamples; t2++) {
                                 const uint32_t v = tab[t2];
                                 tl += (strict[u] ? v < w_bits : v <= w_bits) ? 1 : 0;
                             }
                             const int base0 = lo[u];
-                            if (tl > 0) lo[u] = base0 + (int)(((uint32_t)len * (uint32_t)tl) >> 4) + 1;
-                            if (tl < 15) hi[u] = base0 + (int)(((uint32_t)len * (uint32_t)(tl + 1)) >> 4);
+                            if (tl > 0) lo[u] = base0 + (int)(((uint32_t)len * (uint32_t)tl) >> kSampleShift) + 1;
+                            if (tl < kSamples - 1) hi[u] = base0 + (int)(((uint32_t)len * (uint32_t)(tl + 1)) >> kSampleShift);
                         }
                     }
                     for (;;) {
@@ -999,13 +1000,13 @@ int query_block(const QueryArgs& a_in, hipStream_t s) {
     } while (0)
         // The kernel's time is chains of dependent reads, so what counts is how many items a CU holds: as
         // many as LDS lets in, with the registers that leaves (wavefronts per SIMD = the second template
-        // argument).  Where few promotions are expected and LDS lets ten or more items in, the workgroup
+        // argument).  Where few promotions are expected and LDS lets twelve or more items in, the workgroup
         // is two wavefronts instead of four: half the threads per item, more items within the same
         // registers (1M x 128, 17858-point partitions, four wavefronts: 5 / 6 / 7 / 8 workgroups per CU
-        // 275 / 301 / 309 / 287 k queries/s, eight spilling; two wavefronts, ten workgroups: 326 k; with
-        // nine or fewer items per CU -- partitions above ~22 k points -- two wavefronts lose: 287 against
-        // 300 k at 26316 points, 224 against 279 k at 35715).
-        const bool narrow = 4 * a.M * a.L <= kNarrowThreads && y.promo_cap <= 128 && fit >= 10;
+        // 275 / 301 / 309 / 287 k queries/s, eight spilling; two wavefronts, ten / twelve / thirteen
+        // workgroups: 326 / 349 / 354 k; with fewer items per CU -- partitions above ~22 k points -- two
+        // wavefronts lose: 287 against 300 k at 26316 points, 224 against 279 k at 35715).
+        const bool narrow = 4 * a.M * a.L <= kNarrowThreads && y.promo_cap <= 128 && fit >= 12;
         int minw = narrow ? (fit * (kNarrowThreads / 64) + 3) / 4 : fit;      // wavefronts per SIMD
         minw = minw >= 7 ? 7 : (minw < 3 ? 3 : minw);
         if (narrow) {
