@@ -510,6 +510,10 @@ __global__ __launch_bounds__(NT, MINW) void traverse_block_kernel(QueryArgs a, B
         if (np > (uint32_t)y.promo_max || misc[kEventCount] + np > (uint32_t)y.event_cap) {
             bool minimal = true;
             for (int s2 = 0; s2 < S; s2++) minimal = minimal && s_stride[s2] <= 1;
+            // Every thread has read the two counts and the strides before any of them is changed
+            // below: a wavefront that came late would otherwise see the halved strides (or the
+            // cleared count), decide differently and run the epoch the others are undoing.
+            __syncthreads();
             if (minimal && np <= (uint32_t)y.promo_cap && misc[kEventCount] + np <= (uint32_t)y.event_cap) {
                 // cannot go smaller; the tables still hold it
             } else if (minimal) {

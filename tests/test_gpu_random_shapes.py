@@ -9,7 +9,7 @@ import numpy as np
 import pytest
 import torch
 
-from util import engine_index, engine_project, set_agreement
+from util import assert_ids_agree_up_to_rounding, engine_index, engine_project
 
 pytestmark = pytest.mark.gpu
 
@@ -50,6 +50,21 @@ def _points(rng, n, nq, dim, kind):
 # DCIH_RANDOM_SHAPES=<count> widens the sweep for a one-off soak
 @pytest.mark.parametrize("seed", range(int(os.environ.get("DCIH_RANDOM_SHAPES", "150"))))
 def test_random_shape(gpu, oracle, seed):
+    _run_shape(gpu, oracle, seed)
+
+
+# Shapes from wider sweeps that showed something: 1469 has neighbours 1e-7 apart (relative),
+# whose order depends on how a float32 distance is summed; 14569 (one dimension, every
+# projection the same up to sign, windows wider than the promotion tables like at once)
+# makes the batch kernel undo epochs down to the smallest, where its wavefronts once
+# disagreed on whether to undo (run several times: that depended on their timing).
+@pytest.mark.parametrize("seed,times", [(1469, 1), (14569, 6)])
+def test_shapes_that_failed_once(gpu, oracle, seed, times):
+    for _ in range(times):
+        _run_shape(gpu, oracle, seed)
+
+
+def _run_shape(gpu, oracle, seed):
     from dciknn_cuda_amd import _capi
     rng = np.random.default_rng(1000 + seed)
     M, L, n, B, T, k, outer, max_cand, dim, kind = _shape(rng)
@@ -107,7 +122,8 @@ def test_random_shape(gpu, oracle, seed):
         if traversal == "step":
             np.testing.assert_array_equal(ctr[:, 0], rc[:, 0], err_msg="visits " + tag)
         np.testing.assert_allclose(dists, ref["dists"], rtol=1e-5, atol=1e-6, err_msg=tag)
-        if kind == "normal" or kind == "far":     # no exact distance ties: ids must agree
-            assert set_agreement(ids, ref["ids"]) == 1.0, tag
+        if kind == "normal" or kind == "far":     # no exact distance ties: ids agree, up to
+            # pairs nearer to each other than a float32 distance resolves ("far": 1e-7 apart)
+            assert_ids_agree_up_to_rounding(ids, ref["ids"], X, Q, 1e-5, tag)
         else:                                     # ties: same (id present / absent) pattern
             np.testing.assert_array_equal(ids < 0, ref["ids"] < 0, err_msg=tag)

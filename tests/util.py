@@ -12,6 +12,21 @@ def set_agreement(ids_a, ids_b):
     return hit / ids_a.size
 
 
+def assert_ids_agree_up_to_rounding(ids, ref_ids, X, Q, rtol, tag=""):
+    """Rows of ids and ref_ids hold the same points, except where the points that
+    differ lie within rtol (relative) of one another: two candidates that close
+    at the k-th place swap with the summation order of a float32 distance."""
+    for q, (a, b) in enumerate(zip(np.asarray(ids), np.asarray(ref_ids))):
+        sa, sb = set(a.tolist()), set(b.tolist())
+        if sa == sb:
+            continue
+        assert len(sa) == len(sb) and -1 not in (sa ^ sb), "%s query %d: %s" % (tag, q, sorted(sa ^ sb))
+        q64 = Q[q].astype(np.float64)
+        d = {i: np.sqrt(((X[i].astype(np.float64) - q64) ** 2).sum()) for i in sa ^ sb}
+        lo, hi = min(d.values()), max(d.values())
+        assert hi - lo <= rtol * hi, "%s query %d: the rows differ in %s" % (tag, q, d)
+
+
 def engine_index(dci):
     """(skeys, sids) of a built DCI instance as numpy arrays [I][N]."""
     from dciknn_cuda_amd import _capi
