@@ -548,6 +548,8 @@ static int query_impl(dcih_index* h, int dim, int num_queries, const float* d_qu
     a.mode = h->traversal; a.item_list = nullptr; a.item_count = nullptr; a.dense = nullptr;
     a.xcds = h->xcds; a.q_first = 0; a.q_count = num_queries;
     a.dense_items = nullptr; a.dense_count = nullptr; a.dense_cap = 0;
+    a.wide_items = nullptr; a.wide_count = nullptr; a.wide_cap = 0;
+    a.block_list = nullptr; a.block_list_count = nullptr; a.full_tables = 0;
     a.dense_min_promos = h->dense_min_promos;
     a.phase_ticks = h->d_phase_ticks;
     // the hints describe where traversals of one query shape stop; forget them when it
@@ -633,7 +635,10 @@ static int query_impl(dcih_index* h, int dim, int num_queries, const float* d_qu
     const bool dense_lists = h->traversal == 0 && h->dense_min_promos > 0 && !blind &&
                              dense_traversal_supported(a, nullptr) && block_traversal_supported(a, nullptr);
     const size_t dense_bytes = dense_lists ? align_up((size_t)h->xcds * a.dense_cap * sizeof(int32_t)) : 0;
-    int rc = get_ws(qp_bytes + part_bytes + gs_bytes + redo_bytes + 256 + dense_bytes);
+    // (the second pass may have to take every item, up to what one launch of 256-thread workgroups covers)
+    a.wide_cap = std::min((int64_t)num_queries * block_size, (int64_t)1 << 23);
+    const size_t wide_bytes = align_up((size_t)a.wide_cap * sizeof(int32_t));
+    int rc = get_ws(qp_bytes + part_bytes + gs_bytes + redo_bytes + 256 + dense_bytes + wide_bytes);
     if (rc) return rc;
     char* base = ws_base;
     float* d_qproj = (float*)base;
@@ -644,6 +649,8 @@ static int query_impl(dcih_index* h, int dim, int num_queries, const float* d_qu
     a.redo_count = (uint32_t*)(base + qp_bytes + part_bytes + gs_bytes + redo_bytes);
     a.dense_count = a.redo_count + 1;         // one length per die, cleared together with redo_count
     a.dense_items = dense_lists ? (int32_t*)(base + qp_bytes + part_bytes + gs_bytes + redo_bytes + 256) : nullptr;
+    a.wide_count = a.redo_count + kListCountWords - 1;      // (the last of the list lengths that are cleared together)
+    a.wide_items = (int32_t*)(base + qp_bytes + part_bytes + gs_bytes + redo_bytes + 256 + dense_bytes);
 
     mark(h, DCIH_T_QPROJECT, 0, s);
     rc = project(h->d_dirs, I, d_query, num_queries, dim, d_qproj, num_queries, s);

@@ -79,12 +79,25 @@ struct QueryArgs {
     uint32_t* dense_count;   // [xcds]
     int64_t dense_cap;
     int dense_min_promos;    // promotions per (query, partition) from which the dense kernel is the cheaper one
+    // second pass of the batch kernel: items that outgrow its compact per-item tables are listed and
+    // taken up again by the variant with the full tables
+    int32_t* wide_items;     // null, or [wide_cap]
+    uint32_t* wide_count;
+    int64_t wide_cap;
+    const int32_t* block_list;        // null = the launch covers queries q_first .. q_first + q_count; else workgroup w takes block_list[w]
+    const uint32_t* block_list_count; // ... for w below this number
+    int full_tables;         // 1: the batch kernel keeps its per-point flags as bits whatever the shape
     int xcds;                // accelerator dies of the device (each has an L2 of its own)
     int q_first, q_count;    // batch kernel: the queries one launch covers
     int32_t* out_ids;        // [nq][k]
     float* out_dists;        // [nq][k]; blind: null, or the promoting steps as floats
     float* dense;            // null, or [nq][N]: the step-by-step kernel stores every candidate's score here instead of keeping a top-k
 };
+// The query scratch keeps its list lengths in 64 consecutive words that one kernel clears: the
+// step-by-step kernel's redo list, one hand-over list per die (up to 32), and in the last word
+// the batch kernel's second-pass list.
+constexpr int kListCountWords = 64;
+
 // Work order of the batch kernel.  Workgroups go to the XCDs round-robin by their
 // number and every XCD has an L2 of its own, so XCD x is given the partitions x,
 // x + X, ... and works through them one after the other, all queries of a

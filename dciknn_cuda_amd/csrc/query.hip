@@ -406,7 +406,7 @@ int query(const QueryArgs& a_in, hipStream_t s, hipEvent_t* ev, bool* ran) {
         // the dense lists' lengths follow the hand-over list's
         const int64_t cells = a.counters ? (int64_t)a.nq * 4 : 0;
         hipLaunchKernelGGL(zero_u64_kernel, dim3((unsigned)max((int64_t)1, min((int64_t)1024, (cells + 255) / 256))),
-                           dim3(256), 0, s, a.counters, cells, a.redo_count, 1 + a.xcds);
+                           dim3(256), 0, s, a.counters, cells, a.redo_count, kListCountWords);
     }
     if (ev) (void)hipEventRecord(ev[0], s);
     a.item_list = nullptr;

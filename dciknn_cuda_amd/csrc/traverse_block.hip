@@ -33,6 +33,16 @@
 // many points at once is dropped and retried smaller.  Whatever does not fit the
 // fixed LDS tables is handed to the step-by-step kernel through a redo list, so
 // results never depend on which kernel produced them.
+//
+// Two layouts of an item's LDS state.  The full one keeps three kinds of flags as
+// bits per point of the partition (accepted as a candidate; promoted under composite
+// m) and runs as two or four wavefronts per item.  Where a stop is expected to take
+// few promotions (the smallest tables) and the 2 m L streams fit one wavefront, the
+// compact one keeps those flags as members of one small hashed set, so an item's
+// LDS no longer grows with the partition, and runs as ONE wavefront per item: twice
+// as many items per CU, which is what the kernel's time depends on (chains of
+// dependent reads).  The few items that promote more than the set takes are listed
+// and taken up again by a second launch with the full layout.
 #include <cmath>
 #include <type_traits>
 
@@ -52,12 +62,15 @@ constexpr int kSamples = 1 << kSampleShift;
 enum Misc {   // 32-bit scalars shared by the workgroup
     kPromoCount = 0, kEventCount, kAccCount, kFail, kStop, kC0, kStopStepLo, kStopStepHi,
     kArmedLo, kArmedHi, kScannedLo, kScannedHi, kArmed, kNumCand, kTopN, kProbes, kHintSteps, kHintPromos,
-    kFirstJump, kPromoAimBits, kInvLBits, kNeedBits, kItem, kMiscWords
+    kFirstJump, kPromoAimBits, kInvLBits, kNeedBits, kItem, kSetMarked, kMiscWords
 };
 
 struct BlockLayout {
     int seen_words;   // one bit per point of the partition
     int flag_words;   // seen bits + per composite the points it has promoted: (M + 1) * seen_words
+    int set_slots;    // 0, or: instead of those bits, one hashed set of this many words that holds the
+                      // (composite, point) pairs promoted so far and the points accepted as candidates
+    int set_limit;    // promotions an item may make before that set is too full (the item is then redone)
     int off_idx;      // per simple index: p, qp, and the visited run as packed 16-bit pairs (4 * I words)
     int off_stream;   // per stream: consumed, previous, total, stride, composite number (5 * 2I words)
     int off_comp;     // per composite: rho bits, K, active, previous K, sum of inverse priorities, scan flag (6 * M words)
@@ -69,6 +82,17 @@ struct BlockLayout {
     int sort_cap;     // power of two >= kcap + 128: top-k plus one batch of candidates
     size_t lds_bytes;
 };
+
+constexpr int kSetSlots = 384;
+constexpr uint32_t kSetEmpty = 0xffffffffu;
+constexpr uint32_t kSetSeenTag = 63u << 26;       // composites are tagged 0 .. M - 1 <= 61
+
+// Where few promotions are expected per item (the smallest tables) and the streams fit one
+// wavefront, an item is one wavefront and its per-point flags a small hashed set: LDS per
+// item no longer grows with the partition, and twice as many items fit a CU.
+bool block_layout_compact(const QueryArgs& a, int promo_cap) {
+    return !a.full_tables && promo_cap <= 128 && 2 * a.M * a.L <= 64 && a.M <= 62;
+}
 
 BlockLayout make_block_layout(const QueryArgs& a) {
     BlockLayout y;
@@ -93,7 +117,10 @@ BlockLayout make_block_layout(const QueryArgs& a) {
     y.promo_cap = 128;
     while ((double)y.promo_cap < 2.0 * expected && y.promo_cap < 2048) y.promo_cap <<= 1;
     y.promo_max = y.promo_cap * 5 / 8;
-    y.event_cap = 2 * y.promo_cap;
+    const bool compact = block_layout_compact(a, y.promo_cap);
+    y.set_slots = compact ? kSetSlots : 0;
+    y.set_limit = kSetSlots * 7 / 16;     // every promotion adds at most two entries: the set stays under 7/8 full
+    y.event_cap = compact ? y.promo_cap : 2 * y.promo_cap;
     y.sort_cap = 64;           // top-k plus a batch of at least 48 new candidates
     while (y.sort_cap < a.kcap + 48) y.sort_cap <<= 1;
     // the accepted candidates of a replay share the room of the priority samples and the
@@ -107,13 +134,13 @@ BlockLayout make_block_layout(const QueryArgs& a) {
     y.off_events = o;   o += y.event_cap * 8;
     y.off_sort = o;     o += y.sort_cap * 8;
     y.off_flags = o;
-    y.lds_bytes = (size_t)o + (size_t)y.flag_words * 4;
+    y.lds_bytes = (size_t)o + (size_t)(compact ? y.set_slots : y.flag_words) * 4;
     return y;
 }
 
 // MINW = waves per SIMD the register allocation must leave room for: LDS decides how
 // many workgroups fit a CU, and the kernel should not be the tighter limit.
-template <int NT, int MINW>
+template <int NT, int MINW, bool COMPACT>
 __global__ __launch_bounds__(NT, MINW) void traverse_block_kernel(QueryArgs a, BlockLayout y) {
     extern __shared__ __align__(16) unsigned char smem[];
     uint32_t* misc = reinterpret_cast<uint32_t*>(smem);
@@ -140,6 +167,38 @@ __global__ __launch_bounds__(NT, MINW) void traverse_block_kernel(QueryArgs a, B
     unsigned long long* sortbuf = reinterpret_cast<unsigned long long*>(smem + y.off_sort);
     uint32_t* seen = reinterpret_cast<uint32_t*>(smem + y.off_flags);
     uint32_t* marked = seen + y.seen_words;          // [M][seen_words]: promoted under composite m in an accepted epoch
+    // The compact layout keeps both kinds of flags as members of one open-addressed set in the same
+    // place: (composite << 26 | point) for a promotion, (63 << 26 | point) for an accepted candidate.
+    // The set never fills (set_limit), so every probe sequence ends at an empty word; the probe
+    // count is bounded all the same.
+    const uint32_t set_slots = (uint32_t)y.set_slots;
+    // (false at compile time in the variants for the full tables; in the others left for the kernel to
+    //  test: told at compile time, the compiler duplicates the phases' code around the set's probe loops
+    //  and the seven-wavefront variant keeps 80 bytes per lane in scratch instead of 16)
+    const bool compact = COMPACT && set_slots != 0;
+    uint32_t* const hset = seen;
+    auto set_home = [&](uint32_t key) { return (((key * 0x9E3779B1u) >> 16) * set_slots) >> 16; };
+    auto set_has = [&](uint32_t key) {
+        uint32_t h = set_home(key);
+        for (uint32_t probe = 0; probe < set_slots; probe++) {
+            const uint32_t v = hset[h];
+            if (v == key) return true;
+            if (v == kSetEmpty) return false;
+            h = h + 1 == set_slots ? 0 : h + 1;
+        }
+        return false;
+    };
+    auto set_add = [&](uint32_t key) {        // true if the key was not a member yet
+        uint32_t h = set_home(key);
+        for (uint32_t probe = 0; probe < set_slots; probe++) {
+            const uint32_t v = atomicCAS(&hset[h], kSetEmpty, key);
+            if (v == kSetEmpty) return true;
+            if (v == key) return false;
+            h = h + 1 == set_slots ? 0 : h + 1;
+        }
+        misc[kFail] = 4;
+        return false;
+    };
 
     // The thread numbers are made opaque again at the start of every phase (fresh_thread_ids):
     // otherwise the compiler computes each phase's lane groupings and per-thread addresses once,
@@ -187,8 +246,15 @@ __global__ __launch_bounds__(NT, MINW) void traverse_block_kernel(QueryArgs a, B
     // which (partition, query) this workgroup works on: see block_item (one partition's
     // slices stay in the L2 of the XCD that works through its queries)
     int b, qi;
-    if (!block_item((int64_t)blockIdx.x, a.xcds, a.B, a.q_count, b, qi)) return;
-    qi += a.q_first;
+    if (a.block_list) {       // second pass: the listed items
+        if (blockIdx.x >= *a.block_list_count) return;
+        const int32_t listed = a.block_list[blockIdx.x];
+        b = listed % a.B;
+        qi = listed / a.B;
+    } else {
+        if (!block_item((int64_t)blockIdx.x, a.xcds, a.B, a.q_count, b, qi)) return;
+        qi += a.q_first;
+    }
     const int64_t item = (int64_t)qi * a.B + b;
     const int64_t off = (int64_t)b * a.ppb;
     const int n = (int)min(a.N - off, a.ppb);
@@ -231,6 +297,30 @@ __global__ __launch_bounds__(NT, MINW) void traverse_block_kernel(QueryArgs a, B
         hand_to_dense();
         return;
     }
+    // An item that outgrows the compact tables goes to the second pass, anything else the kernel
+    // cannot finish (and what the second pass's list has no room for) to the step-by-step kernel.
+    auto hand_back = [&]() {
+        if (threadIdx.x == 0) {
+            bool listed = false;
+            if (misc[kFail] == 4 && a.wide_items) {
+                const uint32_t slot = atomicAdd(a.wide_count, 1u);
+                listed = (int64_t)slot < a.wide_cap;
+                if (listed) a.wide_items[slot] = (int32_t)misc[kItem];
+            }
+            if (!listed) {
+                const uint32_t slot = atomicAdd(a.redo_count, 1u);
+                a.redo_items[slot] = (int32_t)misc[kItem];
+            }
+        }
+    };
+    // Where stops in this partition usually need more promotions than the compact tables take,
+    // the item goes to the second pass at once.
+    if (COMPACT && a.wide_items && hint_promos > 0.75f * (float)y.set_limit) {
+        if (threadIdx.x == 0) misc[kFail] = 4;
+        __syncthreads();
+        hand_back();
+        return;
+    }
     const int T = a.T;
     // d / T for 0 <= d < 65536 (positions inside a partition) by one multiply-high:
     // exact because the error of the rounded-up reciprocal stays below 2^-16 < 1/T
@@ -238,7 +328,8 @@ __global__ __launch_bounds__(NT, MINW) void traverse_block_kernel(QueryArgs a, B
     auto div_T = [&](int d) { return T > 1 ? (int)__umulhi((uint32_t)d, T_magic) : d; };
 
     // ---- set-up ---------------------------------------------------------------
-    for (int w = tid; w < y.flag_words; w += NT) seen[w] = 0;
+    if (compact) { for (int w = tid; w < y.set_slots; w += NT) hset[w] = kSetEmpty; }
+    else { for (int w = tid; w < y.flag_words; w += NT) seen[w] = 0; }
     uint32_t probes = 0;
     {   // positioning search (:279-297): first position whose key is not below qp,
         // one group of lanes per simple index
@@ -406,7 +497,7 @@ __global__ __launch_bounds__(NT, MINW) void traverse_block_kernel(QueryArgs a, B
                     if (((w >> ((e & 1) * 16)) & 0xffffu) != 0u) continue;
                     // the point standing at that place of the first index's slice
                     const uint32_t local = (uint32_t)(a.sids[first_row + first + e] - (int32_t)off);
-                    if ((marked_m[local >> 5] >> (local & 31u)) & 1u) continue;
+                    if (compact ? set_has(local | ((uint32_t)m << 26)) : (bool)((marked_m[local >> 5] >> (local & 31u)) & 1u)) continue;
                     const uint32_t slot = atomicAdd(&misc[kPromoCount], 1u);
                     if (slot < (uint32_t)y.promo_cap) promo[slot] = local | ((uint32_t)m << 26);
                 }
@@ -417,7 +508,8 @@ __global__ __launch_bounds__(NT, MINW) void traverse_block_kernel(QueryArgs a, B
     auto mark_promotions = [&](uint32_t np) {
         for (uint32_t j = tid; j < np; j += NT) {
             const uint32_t local = promo[j] & 0x3ffffffu, m = promo[j] >> 26;
-            atomicOr(&marked[m * y.seen_words + (local >> 5)], 1u << (local & 31u));
+            if (compact) set_add(promo[j]);
+            else atomicOr(&marked[m * y.seen_words + (local >> 5)], 1u << (local & 31u));
         }
     };
     bool shrunk = false;        // the previous epoch was undone
@@ -532,6 +624,12 @@ __global__ __launch_bounds__(NT, MINW) void traverse_block_kernel(QueryArgs a, B
             }
         }
 
+        if (compact && misc[kSetMarked] + np > (uint32_t)y.set_limit) {     // (the same for every thread: last written before the barriers above)
+            __syncthreads();
+            if (tid == 0) misc[kFail] = 4;
+            __syncthreads();
+            break;
+        }
         mark_promotions(np);      // the epoch stands: later scans skip its promotions
 
         // ---- 4. exact step of every promotion -----------------------------------
@@ -692,7 +790,7 @@ __global__ __launch_bounds__(NT, MINW) void traverse_block_kernel(QueryArgs a, B
             const uint32_t ev_t = (uint32_t)(ev >> 32);          // steps fit 32 bits (checked by the host)
             const uint32_t ev_e = (uint32_t)ev;
             const uint32_t local = ev_e & 0x1ffffffu;
-            const bool pre = have && ((seen[local >> 5] >> (local & 31u)) & 1u);
+            const bool pre = have && (compact ? set_has(kSetSeenTag | local) : (bool)((seen[local >> 5] >> (local & 31u)) & 1u));
             bool dup = false;      // the same point earlier in the list (promoted under another composite)
             for (int j = 0; j + 1 < ne; j++) {
                 const uint32_t lj = (uint32_t)__builtin_amdgcn_readlane((int)local, j);
@@ -738,7 +836,8 @@ __global__ __launch_bounds__(NT, MINW) void traverse_block_kernel(QueryArgs a, B
                 const uint32_t slot = nacc0 + (uint32_t)__popcll(take & ((1ull << lane) - 1ull));
                 acc[slot] = local;
                 if (a.blind) acc_step[slot] = ev_t;
-                atomicOr(&seen[local >> 5], 1u << (local & 31u));
+                if (compact) set_add(kSetSeenTag | local);
+                else atomicOr(&seen[local >> 5], 1u << (local & 31u));
             }
             // keep what is not settled yet
             const int keep = stop ? 0 : ne - idx;
@@ -753,6 +852,7 @@ __global__ __launch_bounds__(NT, MINW) void traverse_block_kernel(QueryArgs a, B
                 misc[kStop] = stop ? 1u : 0u;
                 misc[kStopStepLo] = (uint32_t)kk_star; misc[kStopStepHi] = (uint32_t)(kk_star >> 32);
                 misc[kPromoCount] = 0;
+                misc[kSetMarked] += np;
             }
         } else if (ne > kWave && tid == 0) {
             long long c0 = (long long)misc[kC0];
@@ -776,8 +876,10 @@ __global__ __launch_bounds__(NT, MINW) void traverse_block_kernel(QueryArgs a, B
                     const uint32_t e = (uint32_t)events[idx];
                     const uint32_t local = e & 0x1ffffffu;
                     const uint32_t bit = 1u << (local & 31);
-                    if (!(seen[local >> 5] & bit)) {
-                        seen[local >> 5] |= bit;
+                    bool fresh;
+                    if (compact) fresh = set_add(kSetSeenTag | local);
+                    else { fresh = !(seen[local >> 5] & bit); seen[local >> 5] |= bit; }
+                    if (fresh) {
                         if (a.blind) acc_step[nacc] = (uint32_t)t;
                         acc[nacc++] = local;
                         ncand++;
@@ -806,6 +908,7 @@ __global__ __launch_bounds__(NT, MINW) void traverse_block_kernel(QueryArgs a, B
             misc[kStop] = stop ? 1u : 0u;
             misc[kStopStepLo] = (uint32_t)kk_star; misc[kStopStepHi] = (uint32_t)(kk_star >> 32);
             misc[kPromoCount] = 0;
+            misc[kSetMarked] += np;
         }
         __syncthreads();
         PHASE_END(6);
@@ -906,10 +1009,7 @@ __global__ __launch_bounds__(NT, MINW) void traverse_block_kernel(QueryArgs a, B
             atomicAdd(&a.phase_ticks[11 + min(3u, misc[kFail])], 1ull);
             a.phase_ticks[15] = ((unsigned long long)item << 32) | ((unsigned long long)misc[kEventCount] << 16) | misc[kPromoCount];
         }
-        if (tid == 0) {
-            const uint32_t slot = atomicAdd(a.redo_count, 1u);
-            a.redo_items[slot] = (int32_t)item;
-        }
+        hand_back();
         return;
     }
 
@@ -974,12 +1074,69 @@ bool block_traversal_supported(const QueryArgs& a, size_t* lds_bytes) {
     return y.lds_bytes <= 160 * 1024 - 512;
 }
 
+// One launch of the kernel variant that suits the layout: `items` workgroups.
+static int launch_block(const QueryArgs& a, const BlockLayout& y, int64_t items, hipStream_t s) {
+    const int fit = (int)(160 * 1024 / y.lds_bytes);      // workgroups per CU by LDS
+#define DCIH_LAUNCH(NT, MW)                                                                        \
+    do {                                                                                           \
+        static DeviceOnce once;                                                                    \
+        const int rc_attr = once.run([]() -> int {                                                 \
+            DCIH_HIP(hipFuncSetAttribute((const void*)traverse_block_kernel<NT, MW, NT == kWave>,  \
+                                         hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024)); \
+            return 0;                                                                              \
+        });                                                                                        \
+        if (rc_attr) return rc_attr;                                                               \
+        hipLaunchKernelGGL((traverse_block_kernel<NT, MW, NT == kWave>), dim3((unsigned)items),    \
+                           dim3(NT), y.lds_bytes, s, a, y);                                        \
+    } while (0)
+    // The kernel's time is chains of dependent reads, so what counts is how many items a CU holds: as
+    // many as LDS lets in, with the registers that leaves (wavefronts per SIMD = the second template
+    // argument).  Measured on 1M x 128, 17242-point partitions, thread_size 2: four wavefronts per item,
+    // 5 / 6 / 7 workgroups per CU 275 / 301 / 309 k queries/s; two wavefronts, ten / twelve / thirteen
+    // workgroups 326 / 349 / 354 k (with fewer items per CU -- partitions above ~22 k points -- two
+    // wavefronts lose to four: 287 against 300 k at 26316 points); one wavefront with the full layout,
+    // thirteen items, 260 k; one wavefront with the compact layout, twenty-six items, 366 k.
+    if (y.set_slots) {      // compact layout: one wavefront per item
+        const int w = fit >= 25 ? 7 : (fit >= 21 ? 6 : (fit >= 17 ? 5 : 4));
+        if (w == 7) DCIH_LAUNCH(kWave, 7); else if (w == 6) DCIH_LAUNCH(kWave, 6);
+        else if (w == 5) DCIH_LAUNCH(kWave, 5); else DCIH_LAUNCH(kWave, 4);
+        DCIH_HIP(hipGetLastError());
+        return 0;
+    }
+    const bool narrow = 4 * a.M * a.L <= kNarrowThreads && y.promo_cap <= 128 && fit >= 12;
+    int minw = narrow ? (fit * (kNarrowThreads / 64) + 3) / 4 : fit;      // wavefronts per SIMD
+    minw = minw >= 7 ? 7 : (minw < 3 ? 3 : minw);
+    if (narrow) {
+        if (minw >= 7) DCIH_LAUNCH(kNarrowThreads, 7); else if (minw == 6) DCIH_LAUNCH(kNarrowThreads, 6);
+        else if (minw == 5) DCIH_LAUNCH(kNarrowThreads, 5); else if (minw == 4) DCIH_LAUNCH(kNarrowThreads, 4);
+        else DCIH_LAUNCH(kNarrowThreads, 3);
+    } else {
+        if (minw >= 7) DCIH_LAUNCH(kBlockThreads, 7); else if (minw == 6) DCIH_LAUNCH(kBlockThreads, 6);
+        else if (minw == 5) DCIH_LAUNCH(kBlockThreads, 5); else if (minw == 4) DCIH_LAUNCH(kBlockThreads, 4);
+        else DCIH_LAUNCH(kBlockThreads, 3);
+    }
+#undef DCIH_LAUNCH
+    DCIH_HIP(hipGetLastError());
+    return 0;
+}
+
 int query_block(const QueryArgs& a_in, hipStream_t s) {
     const BlockLayout y = make_block_layout(a_in);
-    const int fit = (int)(160 * 1024 / y.lds_bytes);      // workgroups per CU by LDS
     // as many queries per launch as the launch limit allows (nearly always all of them)
     const int per_launch = block_queries_per_launch(a_in.xcds, a_in.B, a_in.nq);
     if (per_launch < 1) return fail(-4, "query: block_size too large for the batch traversal kernel");
+    // The items that outgrow the compact tables are taken up again with the full ones, if those fit
+    // LDS (else they go to the step-by-step kernel like everything else the kernel hands back).
+    QueryArgs second = a_in;
+    second.full_tables = 1;
+    second.block_list = a_in.wide_items;
+    second.block_list_count = a_in.wide_count;
+    second.wide_items = nullptr;
+    second.q_first = 0;
+    second.q_count = a_in.nq;
+    const BlockLayout y2 = make_block_layout(second);
+    const bool two_passes = y.set_slots != 0 && a_in.wide_items != nullptr && a_in.wide_cap > 0 &&
+                            y2.lds_bytes <= 160 * 1024 - 512;
     // With nothing known yet about where traversals stop, a few queries go ahead in a launch of
     // their own: their stops are on record when the others start, which then size their first
     // epoch from them instead of feeling their way forward (the first resident round of every
@@ -987,43 +1144,16 @@ int query_block(const QueryArgs& a_in, hipStream_t s) {
     const int lead = a_in.hints_cold && a_in.stop_hint && a_in.nq >= 8 * kLeadQueries ? kLeadQueries : 0;
     for (int q0 = 0; q0 < a_in.nq; q0 += (q0 < lead ? lead : per_launch)) {
         QueryArgs a = a_in;
+        if (!two_passes) a.wide_items = nullptr;
         a.q_first = q0;
         a.q_count = q0 < lead ? lead : min(per_launch, a_in.nq - q0);
-        const int64_t items = block_items(a.xcds, a.B, a.q_count);
-#define DCIH_LAUNCH(NT, MW)                                                                        \
-    do {                                                                                           \
-        static DeviceOnce once;                                                                    \
-        const int rc_attr = once.run([]() -> int {                                                 \
-            DCIH_HIP(hipFuncSetAttribute((const void*)traverse_block_kernel<NT, MW>,               \
-                                         hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024)); \
-            return 0;                                                                              \
-        });                                                                                        \
-        if (rc_attr) return rc_attr;                                                               \
-        hipLaunchKernelGGL((traverse_block_kernel<NT, MW>), dim3((unsigned)items),                 \
-                           dim3(NT), y.lds_bytes, s, a, y);                                        \
-    } while (0)
-        // The kernel's time is chains of dependent reads, so what counts is how many items a CU holds: as
-        // many as LDS lets in, with the registers that leaves (wavefronts per SIMD = the second template
-        // argument).  Where few promotions are expected and LDS lets twelve or more items in, the workgroup
-        // is two wavefronts instead of four: half the threads per item, more items within the same
-        // registers (1M x 128, 17858-point partitions, four wavefronts: 5 / 6 / 7 / 8 workgroups per CU
-        // 275 / 301 / 309 / 287 k queries/s, eight spilling; two wavefronts, ten / twelve / thirteen
-        // workgroups: 326 / 349 / 354 k; with fewer items per CU -- partitions above ~22 k points -- two
-        // wavefronts lose: 287 against 300 k at 26316 points, 224 against 279 k at 35715).
-        const bool narrow = 4 * a.M * a.L <= kNarrowThreads && y.promo_cap <= 128 && fit >= 12;
-        int minw = narrow ? (fit * (kNarrowThreads / 64) + 3) / 4 : fit;      // wavefronts per SIMD
-        minw = minw >= 7 ? 7 : (minw < 3 ? 3 : minw);
-        if (narrow) {
-            if (minw >= 7) DCIH_LAUNCH(kNarrowThreads, 7); else if (minw == 6) DCIH_LAUNCH(kNarrowThreads, 6);
-            else if (minw == 5) DCIH_LAUNCH(kNarrowThreads, 5); else if (minw == 4) DCIH_LAUNCH(kNarrowThreads, 4);
-            else DCIH_LAUNCH(kNarrowThreads, 3);
-        } else {
-            if (minw >= 7) DCIH_LAUNCH(kBlockThreads, 7); else if (minw == 6) DCIH_LAUNCH(kBlockThreads, 6);
-            else if (minw == 5) DCIH_LAUNCH(kBlockThreads, 5); else if (minw == 4) DCIH_LAUNCH(kBlockThreads, 4);
-            else DCIH_LAUNCH(kBlockThreads, 3);
-        }
-#undef DCIH_LAUNCH
-        DCIH_HIP(hipGetLastError());
+        const int rc = launch_block(a, y, block_items(a.xcds, a.B, a.q_count), s);
+        if (rc) return rc;
+    }
+    if (two_passes) {
+        const int64_t most = min(a_in.wide_cap, (int64_t)a_in.nq * a_in.B);
+        const int rc = launch_block(second, y2, most, s);
+        if (rc) return rc;
     }
     return 0;
 }
