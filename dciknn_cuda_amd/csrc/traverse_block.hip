@@ -72,7 +72,7 @@ struct BlockLayout {
                       // (composite, point) pairs promoted so far and the points accepted as candidates
     int set_limit;    // promotions an item may make before that set is too full (the item is then redone)
     int off_idx;      // per simple index: p, qp, and the visited run as packed 16-bit pairs (4 * I words)
-    int off_stream;   // per stream: consumed, previous, total, stride, composite number (5 * 2I words)
+    int off_stream;   // per stream: consumed, previous, total, stride (4 * 2I words)
     int off_comp;     // per composite: rho bits, K, active, previous K, sum of inverse priorities, scan flag (6 * M words)
     int off_samp;     // per stream: kSamples - 1 sampled window priorities of the current epoch's range (slot 0 unused)
     int off_promo, off_events, off_acc, off_sort, off_flags;
@@ -101,7 +101,7 @@ BlockLayout make_block_layout(const QueryArgs& a) {
     y.flag_words = (a.M + 1) * y.seen_words;
     int o = kMiscWords * 4;
     y.off_idx = o;      o += 4 * I * 4;
-    y.off_stream = o;   o += 5 * 2 * I * 4;
+    y.off_stream = o;   o += 4 * 2 * I * 4;
     y.off_comp = o;     o += 6 * a.M * 4;
     // small tables keep more workgroups resident per CU; an item that overflows them
     // is redone by the step-by-step kernel
@@ -152,7 +152,6 @@ __global__ __launch_bounds__(NT, MINW) void traverse_block_kernel(QueryArgs a, B
     int* s_cprev = s_c + 2 * a.M * a.L;                               // ... at epoch start
     int* s_ns = s_cprev + 2 * a.M * a.L;                              // windows in the stream
     int* s_stride = s_ns + 2 * a.M * a.L;                             // windows to try next epoch
-    int* s_mof = s_stride + 2 * a.M * a.L;                            // composite the stream belongs to
     uint32_t* s_rho = reinterpret_cast<uint32_t*>(smem + y.off_comp); // per composite
     uint32_t* s_K = s_rho + a.M;
     uint32_t* s_active = s_K + a.M;
@@ -347,7 +346,6 @@ __global__ __launch_bounds__(NT, MINW) void traverse_block_kernel(QueryArgs a, B
             for (int side = 0; side < 2; side++) {
                 s_ns[2 * i + side] = stream_windows(n, T, p, side);
                 s_c[2 * i + side] = 0;
-                s_mof[2 * i + side] = i / a.L;
             }
         }
     }
