@@ -62,7 +62,7 @@ constexpr int kSamples = 1 << kSampleShift;
 enum Misc {   // 32-bit scalars shared by the workgroup
     kPromoCount = 0, kEventCount, kAccCount, kFail, kStop, kC0, kStopStepLo, kStopStepHi,
     kArmedLo, kArmedHi, kScannedLo, kScannedHi, kArmed, kNumCand, kTopN, kProbes, kHintSteps, kHintPromos,
-    kFirstJump, kPromoAimBits, kInvLBits, kNeedBits, kItem, kSetMarked, kMiscWords
+    kFirstJump, kPromoAimBits, kInvLBits, kNeedBits, kItem, kSetMarked, kListCount, kMiscWords
 };
 
 struct BlockLayout {
@@ -444,11 +444,18 @@ __global__ __launch_bounds__(NT, MINW) void traverse_block_kernel(QueryArgs a, B
             const int chunk_shift = (a.N & 7) == 0 ? (int)((off + run_lo) & 7) : 0;
             const int start = run_lo - chunk_shift;
             const int nchunks = (run_hi - start + 7) >> 3;
-            looked_at += (unsigned long long)nchunks * 8ull * (unsigned long long)(a.L - 1);
             const uint16_t* rp = a.rpos + first_row + start;
-            for (int c = tid; c < nchunks; c += NT) {
+            // a point found inside all runs: to the promotion list unless an earlier epoch promoted it
+            auto found = [&](int place) {        // place in the first index's slice
+                const uint32_t local = (uint32_t)(a.sids[first_row + place] - (int32_t)off);
+                if (compact ? set_has(local | ((uint32_t)m << 26)) : (bool)((marked_m[local >> 5] >> (local & 31u)) & 1u)) return;
+                const uint32_t slot = atomicAdd(&misc[kPromoCount], 1u);
+                if (slot < (uint32_t)y.promo_cap) promo[slot] = local | ((uint32_t)m << 26);
+            };
+            // rows [h_begin, h_end) of the position table for chunk c: the fields of `worst` that stay
+            // zero belong to places inside the runs of all those rows (and inside the first index's run)
+            auto test_chunk = [&](int c, int h_begin, int h_end, u16x2 (&worst)[4]) {
                 const int first = start + 8 * c;            // place in the first index's slice of the chunk's first point
-                u16x2 worst[4];
 #pragma unroll
                 for (int r = 0; r < 4; r++) worst[r] = u16x2{0, 0};
                 if (c == 0 || c == nchunks - 1) {            // places before the run's first or past its last
@@ -482,22 +489,88 @@ __global__ __launch_bounds__(NT, MINW) void traverse_block_kernel(QueryArgs a, B
                         }
                     }
                 };
-                int h0 = 1;
-                for (; h0 + 2 <= a.L; h0 += 2) group(h0, std::integral_constant<int, 2>());
-                if (h0 < a.L) group(h0, std::integral_constant<int, 1>());
+                // (rows per group of reads in flight: three where all rows are read in one stage, two in the
+                //  two-stage form -- each measured a per cent or two ahead of the other there)
+                int h0 = h_begin;
+                if (!COMPACT) for (; h0 + 3 <= h_end; h0 += 3) group(h0, std::integral_constant<int, 3>());
+                for (; h0 + 2 <= h_end; h0 += 2) group(h0, std::integral_constant<int, 2>());
+                if (h0 < h_end) group(h0, std::integral_constant<int, 1>());
                 const u16x2 m01 = __builtin_elementwise_min(worst[0], worst[1]);
                 const u16x2 m23 = __builtin_elementwise_min(worst[2], worst[3]);
                 const uint32_t least = __builtin_bit_cast(uint32_t, __builtin_elementwise_min(m01, m23));
-                if (((least - 0x00010001u) & ~least & 0x80008000u) == 0u) continue;     // no 16-bit field is zero
+                return ((least - 0x00010001u) & ~least & 0x80008000u) != 0u;     // some 16-bit field is zero
+            };
+            // Two stages where the composite has many simple indices (one-wavefront variants): about half
+            // of the places survive each row, so after the first 0.6 L rows few are left; those are listed
+            // (their distance from the run's first place, 16 bits, in the room of the priority samples,
+            // which are taken after the scan) and only for them the remaining rows are read, one 2-byte
+            // read per row and place -- far dearer per place than the first stage's, hence not earlier
+            // (1M x 128, L = 10, 17242-point partitions: one stage 365 k queries/s; 3 / 4 / 5 / 6 / 7 rows
+            // in the first stage 331 / 373 / 397 / 398 / 385 k).  The list is emptied whenever the next
+            // round of chunks might overflow it.
+            const int stage_rows = (3 * a.L + 2) / 5;
+            uint16_t* const list = reinterpret_cast<uint16_t*>(s_samp);
+            const int list_cap = 2 * I * kSamples * 2;
+            if (COMPACT && a.L - 1 > stage_rows + 1 && list_cap >= 8 * NT + NT) {
+                auto rest_of_rows = [&](int n_listed) {
+                    for (int j = tid; j < n_listed; j += NT) {
+                        const int place = run_lo + (int)list[j];
+                        bool inside = true;
+                        for (int h0 = 1 + stage_rows; h0 < a.L; h0 += 4) {
+                            uint32_t pos[4];
+#pragma unroll
+                            for (int u = 0; u < 4; u++) {
+                                const int h = min(h0 + u, a.L - 1);
+                                pos[u] = a.rpos[first_row + (int64_t)h * a.N + place];
+                            }
+#pragma unroll
+                            for (int u = 0; u < 4; u++) {
+                                const int h = min(h0 + u, a.L - 1);
+                                inside = inside && ((pos[u] - (lo2[h] & 0xffffu)) & 0xffffu) <= (lm2[h] & 0xffffu);
+                            }
+                        }
+                        if (inside) found(place);
+                    }
+                };
+                unsigned long long listed_total = 0;
+                for (int c0 = 0; c0 < nchunks; c0 += NT) {
+                    const int c = c0 + tid;
+                    if (c < nchunks) {
+                        u16x2 worst[4];
+                        if (test_chunk(c, 1, 1 + stage_rows, worst)) {
+#pragma unroll
+                            for (int e = 0; e < 8; e++) {
+                                const uint32_t w = __builtin_bit_cast(uint32_t, worst[e >> 1]);
+                                if (((w >> ((e & 1) * 16)) & 0xffffu) != 0u) continue;
+                                const uint32_t slot = atomicAdd(&misc[kListCount], 1u);
+                                list[slot] = (uint16_t)(start + 8 * c + e - run_lo);
+                            }
+                        }
+                    }
+                    __syncthreads();
+                    const int n_listed = (int)misc[kListCount];
+                    __syncthreads();          // (every thread has the count before anyone changes it)
+                    if (n_listed > list_cap - 8 * NT || c0 + NT >= nchunks) {
+                        rest_of_rows(n_listed);
+                        listed_total += (unsigned long long)n_listed;
+                        __syncthreads();
+                        if (tid == 0) misc[kListCount] = 0;
+                        __syncthreads();
+                    }
+                }
+                looked_at += (unsigned long long)nchunks * 8ull * (unsigned long long)stage_rows +
+                             listed_total * (unsigned long long)(a.L - 1 - stage_rows);
+                continue;
+            }
+            looked_at += (unsigned long long)nchunks * 8ull * (unsigned long long)(a.L - 1);
+            for (int c = tid; c < nchunks; c += NT) {
+                u16x2 worst[4];
+                if (!test_chunk(c, 1, a.L, worst)) continue;
 #pragma unroll
                 for (int e = 0; e < 8; e++) {
                     const uint32_t w = __builtin_bit_cast(uint32_t, worst[e >> 1]);
                     if (((w >> ((e & 1) * 16)) & 0xffffu) != 0u) continue;
-                    // the point standing at that place of the first index's slice
-                    const uint32_t local = (uint32_t)(a.sids[first_row + first + e] - (int32_t)off);
-                    if (compact ? set_has(local | ((uint32_t)m << 26)) : (bool)((marked_m[local >> 5] >> (local & 31u)) & 1u)) continue;
-                    const uint32_t slot = atomicAdd(&misc[kPromoCount], 1u);
-                    if (slot < (uint32_t)y.promo_cap) promo[slot] = local | ((uint32_t)m << 26);
+                    found(start + 8 * c + e);
                 }
             }
         }
