@@ -720,7 +720,7 @@ __global__ __launch_bounds__(NT, MINW) void traverse_block_kernel(QueryArgs a, B
             // Eight lanes rank one promotion, so 32 promotions are in flight per
             // workgroup; each lane runs the binary searches of up to three streams in
             // lockstep so that their key reads overlap.
-            constexpr int kGroup = 8, kPerLane = 3;
+            constexpr int kGroup = 4, kPerLane = 5;
             const int gl = tid & (kGroup - 1);
             const int group = tid / kGroup;
             for (uint32_t pi = group; pi < np; pi += NT / kGroup) {
@@ -730,24 +730,43 @@ __global__ __launch_bounds__(NT, MINW) void traverse_block_kernel(QueryArgs a, B
                 // farthest of the L windows that hold the point = the last one visited
                 uint32_t w_bits = 0;
                 int w_h = -1, w_side = 0, w_j = 0, w_t = 0;
-                for (int h = gl; h < a.L; h += kGroup) {
-                    const int i = m * a.L + h;
-                    const int pos = (int)a.inv[(int64_t)i * a.N + off + local];
-                    const int p = s_p[i];
-                    const float* key = a.skeys + (int64_t)i * a.N + off;
-                    int side, j, t, kp;
-                    if (pos > p) {
-                        const int d = pos - (p + 1);
-                        side = 1; j = div_T(d); t = d - j * T; kp = p + 1 + j * T;
-                    } else {
-                        const int d = p - pos;
-                        side = 0; j = div_T(d);
-                        const int start = p - T + 1 - j * T;
-                        t = pos - start; kp = max(start, 0);
+                // (a lane's windows four at a time: first all their positions are read, then all their keys)
+                constexpr int kWin = 4;
+                for (int hb = gl; hb < a.L; hb += kGroup * kWin) {
+                    int pos[kWin];
+#pragma unroll
+                    for (int u = 0; u < kWin; u++) {
+                        const int h = min(hb + u * kGroup, a.L - 1);
+                        pos[u] = (int)a.inv[(int64_t)(m * a.L + h) * a.N + off + local];
                     }
-                    probes++;
-                    const uint32_t bits = __builtin_bit_cast(uint32_t, fabsf(key[kp] - s_qp[i]));
-                    if (w_h < 0 || bits >= w_bits) { w_bits = bits; w_h = h; w_side = side; w_j = j; w_t = t; }
+                    int side[kWin], j[kWin], t[kWin];
+                    float kv[kWin];
+#pragma unroll
+                    for (int u = 0; u < kWin; u++) {
+                        const int h = min(hb + u * kGroup, a.L - 1);
+                        const int i = m * a.L + h;
+                        const int p = s_p[i];
+                        const float* key = a.skeys + (int64_t)i * a.N + off;
+                        int kp;
+                        if (pos[u] > p) {
+                            const int d = pos[u] - (p + 1);
+                            side[u] = 1; j[u] = div_T(d); t[u] = d - j[u] * T; kp = p + 1 + j[u] * T;
+                        } else {
+                            const int d = p - pos[u];
+                            side[u] = 0; j[u] = div_T(d);
+                            const int start = p - T + 1 - j[u] * T;
+                            t[u] = pos[u] - start; kp = max(start, 0);
+                        }
+                        kv[u] = key[kp];
+                    }
+#pragma unroll
+                    for (int u = 0; u < kWin; u++) {
+                        const int h = hb + u * kGroup;
+                        if (h >= a.L) continue;
+                        probes++;
+                        const uint32_t bits = __builtin_bit_cast(uint32_t, fabsf(kv[u] - s_qp[m * a.L + h]));
+                        if (w_h < 0 || bits >= w_bits) { w_bits = bits; w_h = h; w_side = side[u]; w_j = j[u]; w_t = t[u]; }
+                    }
                 }
                 auto farthest_of_two = [&](auto width) {      // (lane exchanges by immediate patterns: no address registers)
                     constexpr int O = decltype(width)::value;
@@ -759,14 +778,15 @@ __global__ __launch_bounds__(NT, MINW) void traverse_block_kernel(QueryArgs a, B
                     const bool take = oh >= 0 && (w_h < 0 || ob > w_bits || (ob == w_bits && oh > w_h));
                     if (take) { w_bits = ob; w_h = oh; w_side = os; w_j = oj; w_t = ot; }
                 };
-                static_assert(kGroup == 8, "three exchange levels");
-                farthest_of_two(std::integral_constant<int, 4>());
-                farthest_of_two(std::integral_constant<int, 2>());
+                static_assert(kGroup == 8 || kGroup == 4 || kGroup == 2, "exchange levels");
+                if constexpr (kGroup >= 8) farthest_of_two(std::integral_constant<int, 4>());
+                if constexpr (kGroup >= 4) farthest_of_two(std::integral_constant<int, 2>());
                 farthest_of_two(std::integral_constant<int, 1>());
                 // rank of that window = windows of the composite ordered before it
                 uint32_t rank = 0;
                 for (int s0 = gl; s0 < 2 * a.L; s0 += kGroup * kPerLane) {
-                    Stream st[kPerLane];
+                    // (a stream's description is read again from LDS for every probe -- cheap beside the
+                    //  probe's own read -- instead of being held in registers for all the lane's streams)
                     int lo[kPerLane], hi[kPerLane];
                     bool strict[kPerLane];
 #pragma unroll
@@ -777,9 +797,8 @@ __global__ __launch_bounds__(NT, MINW) void traverse_block_kernel(QueryArgs a, B
                         if (s2 >= 2 * a.L) continue;
                         const int h2 = s2 >> 1, side2 = s2 & 1;
                         const int sidx = 2 * (m * a.L + h2) + side2;
-                        st[u] = load_stream(sidx);
                         if (h2 == w_h) {
-                            const bool corner = st[u].p == n - 1 && T >= 2;   // ghost window first
+                            const bool corner = s_p[sidx >> 1] == n - 1 && T >= 2;   // ghost window first
                             if (side2 == w_side) { lo[u] = hi[u] = w_j; continue; }
                             if (corner) { lo[u] = hi[u] = w_side ? 0 : s_ns[sidx]; continue; }
                             strict[u] = w_side == 0;
@@ -811,7 +830,9 @@ __global__ __launch_bounds__(NT, MINW) void traverse_block_kernel(QueryArgs a, B
                             if (lo[u] < hi[u]) {
                                 any = true;
                                 const int mid = (lo[u] + hi[u]) >> 1;
-                                const uint32_t v = stream_prio_bits(st[u], mid);
+                                int sidx = 2 * m * a.L + s0 + u * kGroup;
+                                asm volatile("" : "+v"(sidx));      // (else the description is fetched once, before the loop, and kept)
+                                const uint32_t v = stream_prio_bits(load_stream(sidx), mid);
                                 probes++;
                                 if (strict[u] ? v < w_bits : v <= w_bits) lo[u] = mid + 1; else hi[u] = mid;
                             }
@@ -821,7 +842,9 @@ __global__ __launch_bounds__(NT, MINW) void traverse_block_kernel(QueryArgs a, B
 #pragma unroll
                     for (int u = 0; u < kPerLane; u++) rank += (uint32_t)lo[u];
                 }
-                rank += lane_xor<4>(rank); rank += lane_xor<2>(rank); rank += lane_xor<1>(rank);
+                if constexpr (kGroup >= 8) rank += lane_xor<4>(rank);
+                if constexpr (kGroup >= 4) rank += lane_xor<2>(rank);
+                rank += lane_xor<1>(rank);
                 if (gl == 0) {
                     const uint32_t slot = atomicAdd(&misc[kEventCount], 1u);
                     if (slot < (uint32_t)y.event_cap) events[slot] = pack_event(rank, m, w_t == 0, local);
