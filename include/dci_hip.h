@@ -195,8 +195,9 @@ int dcih_query(dcih_index* h, int dim, int num_queries, const float* d_query,
  * order: the neighbour sets are then the same and the distances agree to 1e-5
  * relative, not in every bit (and neighbours at tied distances may swap places).
  * Every byte of scratch (query projections, per-partition result
- * lists, hand-over list between the two traversal kernels, global visit counters
- * of partitions too large for on-chip memory) comes from one array of
+ * lists, hand-over lists between the traversal kernels and between the batch
+ * kernel's two passes, global visit counters of partitions too large for on-chip
+ * memory) comes from one array of
  * DCIH_NOALLOC_SCRATCH_BYTES that is part of the library's code object, so each
  * GPU the library runs on holds one such array until the process ends.  The call
  * makes no hipMalloc / hipFree and uses no allocating library routine.  A call
