@@ -315,10 +315,15 @@ __global__ void zero_u64_kernel(unsigned long long* p, int64_t n, uint32_t* also
     if (also && blockIdx.x == 0 && (int)threadIdx.x < also_n) also[threadIdx.x] = 0;
 }
 
-int merge_cap(int k) {
+// Words of the merge's sort buffer: room for the k best plus at least as many new entries, and
+// no more than the per-partition lists hold in all (a sort of 2048 words for 590 entries would
+// spend most of its stages on padding).
+int merge_cap(int k, int64_t total) {
     int cap = 2048;
     while (cap < 2 * k) cap <<= 1;
-    return cap;
+    int need = 64;
+    while ((int64_t)need < (int64_t)k + total && need < cap) need <<= 1;
+    return need < cap ? need : cap;
 }
 
 }  // namespace
@@ -451,7 +456,7 @@ int query(const QueryArgs& a_in, hipStream_t s, hipEvent_t* ev, bool* ran) {
     }
     DCIH_HIP(hipGetLastError());
     if (ev) (void)hipEventRecord(ev[3], s);
-    const int cap = merge_cap(a.k);
+    const int cap = merge_cap(a.k, (int64_t)a.B * a.kcap);
     hipLaunchKernelGGL(merge_topk_kernel, dim3((unsigned)a.nq), dim3(kMergeThreads),
                        (size_t)cap * sizeof(unsigned long long), s, a, cap);
     if (ev) (void)hipEventRecord(ev[4], s);
