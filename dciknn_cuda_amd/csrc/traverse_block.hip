@@ -1185,11 +1185,15 @@ static int launch_block(const QueryArgs& a, const BlockLayout& y, int64_t items,
     } while (0)
     // The kernel's time is chains of dependent reads, so what counts is how many items a CU holds: as
     // many as LDS lets in, with the registers that leaves (wavefronts per SIMD = the second template
-    // argument).  Measured on 1M x 128, 17242-point partitions, thread_size 2: four wavefronts per item,
-    // 5 / 6 / 7 workgroups per CU 275 / 301 / 309 k queries/s; two wavefronts, ten / twelve / thirteen
-    // workgroups 326 / 349 / 354 k (with fewer items per CU -- partitions above ~22 k points -- two
-    // wavefronts lose to four: 287 against 300 k at 26316 points); one wavefront with the full layout,
-    // thirteen items, 260 k; one wavefront with the compact layout, twenty-six items, 366 k.
+    // argument).  Full layout: two wavefronts per item where LDS lets ten or more items into a CU (and the
+    // streams fit their lane groups), else four.  Measured on 1M x 128, thread_size 2: 17242-point
+    // partitions, four wavefronts per item, 5 / 6 / 7 workgroups per CU 275 / 301 / 309 k queries/s; two
+    // wavefronts, ten / twelve / thirteen workgroups 326 / 349 / 354 k; with fewer items per CU two
+    // wavefronts lose to four (287 against 300 k at 26316 points, 79.5 against 88.0 k with eight or nine
+    // items at 26316 points, thread_size 3, 5000 iterations); with the 256-entry tables of the reference's
+    // default setting (10000-point partitions, thread_size 10) two wavefronts give 88.4 against 76.0 k.
+    // One wavefront with the full layout, thirteen items, 260 k; one wavefront with the compact layout,
+    // twenty-six items, 366 k.
     if (y.set_slots) {      // compact layout: one wavefront per item
         const int w = fit >= 25 ? 7 : (fit >= 21 ? 6 : (fit >= 17 ? 5 : 4));
         if (w == 7) DCIH_LAUNCH(kWave, 7); else if (w == 6) DCIH_LAUNCH(kWave, 6);
@@ -1197,7 +1201,7 @@ static int launch_block(const QueryArgs& a, const BlockLayout& y, int64_t items,
         DCIH_HIP(hipGetLastError());
         return 0;
     }
-    const bool narrow = 4 * a.M * a.L <= kNarrowThreads && y.promo_cap <= 128 && fit >= 12;
+    const bool narrow = 4 * a.M * a.L <= kNarrowThreads && fit >= 10;
     int minw = narrow ? (fit * (kNarrowThreads / 64) + 3) / 4 : fit;      // wavefronts per SIMD
     minw = minw >= 7 ? 7 : (minw < 3 ? 3 : minw);
     if (narrow) {
