@@ -296,12 +296,13 @@ __global__ __launch_bounds__(NT, MINW) void traverse_block_kernel(QueryArgs a, B
         hand_to_dense();
         return;
     }
-    // An item that outgrows the compact tables goes to the second pass, anything else the kernel
-    // cannot finish (and what the second pass's list has no room for) to the step-by-step kernel.
+    // An item that the compact tables cannot finish (the set full, or the smaller event table) goes
+    // to the second pass, whose tables may hold it; what the full tables cannot finish either (and
+    // what the second pass's list has no room for) goes to the step-by-step kernel.
     auto hand_back = [&]() {
         if (threadIdx.x == 0) {
             bool listed = false;
-            if (misc[kFail] == 4 && a.wide_items) {
+            if (COMPACT && a.wide_items) {
                 const uint32_t slot = atomicAdd(a.wide_count, 1u);
                 listed = (int64_t)slot < a.wide_cap;
                 if (listed) a.wide_items[slot] = (int32_t)misc[kItem];
