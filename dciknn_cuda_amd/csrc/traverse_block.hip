@@ -138,10 +138,9 @@ BlockLayout make_block_layout(const QueryArgs& a) {
     return y;
 }
 
-// MINW = waves per SIMD the register allocation must leave room for: LDS decides how
-// many workgroups fit a CU, and the kernel should not be the tighter limit.
+// One (query qi, partition b) item, by the whole workgroup.
 template <int NT, int MINW, bool COMPACT>
-__global__ __launch_bounds__(NT, MINW) void traverse_block_kernel(QueryArgs a, BlockLayout y) {
+__device__ __forceinline__ void traverse_block_item(const QueryArgs& a, const BlockLayout& y, const int b, const int qi) {
     extern __shared__ __align__(16) unsigned char smem[];
     uint32_t* misc = reinterpret_cast<uint32_t*>(smem);
     int* s_p = reinterpret_cast<int*>(smem + y.off_idx);
@@ -242,18 +241,6 @@ __global__ __launch_bounds__(NT, MINW) void traverse_block_kernel(QueryArgs a, B
     const int I = a.M * a.L;
     const int S = 2 * I;                       // streams
 
-    // which (partition, query) this workgroup works on: see block_item (one partition's
-    // slices stay in the L2 of the XCD that works through its queries)
-    int b, qi;
-    if (a.block_list) {       // second pass: the listed items
-        if (blockIdx.x >= *a.block_list_count) return;
-        const int32_t listed = a.block_list[blockIdx.x];
-        b = listed % a.B;
-        qi = listed / a.B;
-    } else {
-        if (!block_item((int64_t)blockIdx.x, a.xcds, a.B, a.q_count, b, qi)) return;
-        qi += a.q_first;
-    }
     const int64_t item = (int64_t)qi * a.B + b;
     const int64_t off = (int64_t)b * a.ppb;
     const int n = (int)min(a.N - off, a.ppb);
@@ -1146,6 +1133,29 @@ __global__ __launch_bounds__(NT, MINW) void traverse_block_kernel(QueryArgs a, B
     }
 }
 
+// MINW = waves per SIMD the register allocation must leave room for: LDS decides how
+// many workgroups fit a CU, and the kernel should not be the tighter limit.
+// Which (partition, query) a workgroup works on: see block_item (one partition's slices stay
+// in the L2 of the XCD that works through its queries).
+template <int NT, int MINW, bool COMPACT>
+__global__ __launch_bounds__(NT, MINW) void traverse_block_kernel(QueryArgs a, BlockLayout y) {
+    int b, qi;
+    if (!block_item((int64_t)blockIdx.x, a.xcds, a.B, a.q_count, b, qi)) return;
+    traverse_block_item<NT, MINW, COMPACT>(a, y, b, qi + a.q_first);
+}
+// Second pass: the workgroups stride over the list of items the compact variants handed back
+// (its length is only known on the device, so the grid is a fixed number of resident workgroups).
+template <int NT, int MINW>
+__global__ __launch_bounds__(NT, MINW) void traverse_block_list_kernel(QueryArgs a, BlockLayout y) {
+    const uint32_t listed = *a.block_list_count;
+    const uint32_t count = (int64_t)listed < a.wide_cap ? listed : (uint32_t)a.wide_cap;
+    for (uint32_t w = blockIdx.x; w < count; w += gridDim.x) {
+        const int32_t item = a.block_list[w];
+        traverse_block_item<NT, MINW, false>(a, y, item % a.B, item / a.B);
+        __syncthreads();          // the next item reuses the tables
+    }
+}
+
 constexpr int kBlockThreads = 256;
 constexpr int kNarrowThreads = 128;     // workgroups of two wavefronts: more (query, partition) items per CU
 constexpr int kLeadQueries = 32;
@@ -1172,17 +1182,24 @@ bool block_traversal_supported(const QueryArgs& a, size_t* lds_bytes) {
 // One launch of the kernel variant that suits the layout: `items` workgroups.
 static int launch_block(const QueryArgs& a, const BlockLayout& y, int64_t items, hipStream_t s) {
     const int fit = (int)(160 * 1024 / y.lds_bytes);      // workgroups per CU by LDS
-#define DCIH_LAUNCH(NT, MW)                                                                        \
+#define DCIH_LAUNCH_KERNEL(KERNEL, NT, GRID)                                                      \
     do {                                                                                           \
         static DeviceOnce once;                                                                    \
         const int rc_attr = once.run([]() -> int {                                                 \
-            DCIH_HIP(hipFuncSetAttribute((const void*)traverse_block_kernel<NT, MW, NT == kWave>,  \
+            DCIH_HIP(hipFuncSetAttribute((const void*)KERNEL,                                      \
                                          hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024)); \
             return 0;                                                                              \
         });                                                                                        \
         if (rc_attr) return rc_attr;                                                               \
-        hipLaunchKernelGGL((traverse_block_kernel<NT, MW, NT == kWave>), dim3((unsigned)items),    \
-                           dim3(NT), y.lds_bytes, s, a, y);                                        \
+        hipLaunchKernelGGL(KERNEL, dim3((unsigned)(GRID)), dim3(NT), y.lds_bytes, s, a, y);        \
+    } while (0)
+#define DCIH_LAUNCH_COMPACT(MW) DCIH_LAUNCH_KERNEL((traverse_block_kernel<kWave, MW, true>), kWave, items)
+    // (the second pass: as many workgroups as the device holds at a time, striding over the list)
+    const int64_t resident = std::min(items, (int64_t)a.xcds * 32 * std::max(1, fit));
+#define DCIH_LAUNCH(NT, MW)                                                                        \
+    do {                                                                                           \
+        if (a.block_list) DCIH_LAUNCH_KERNEL((traverse_block_list_kernel<NT, MW>), NT, resident);  \
+        else DCIH_LAUNCH_KERNEL((traverse_block_kernel<NT, MW, false>), NT, items);                \
     } while (0)
     // The kernel's time is chains of dependent reads, so what counts is how many items a CU holds: as
     // many as LDS lets in, with the registers that leaves (wavefronts per SIMD = the second template
@@ -1197,8 +1214,8 @@ static int launch_block(const QueryArgs& a, const BlockLayout& y, int64_t items,
     // twenty-six items, 366 k.
     if (y.set_slots) {      // compact layout: one wavefront per item
         const int w = fit >= 25 ? 7 : (fit >= 21 ? 6 : (fit >= 17 ? 5 : 4));
-        if (w == 7) DCIH_LAUNCH(kWave, 7); else if (w == 6) DCIH_LAUNCH(kWave, 6);
-        else if (w == 5) DCIH_LAUNCH(kWave, 5); else DCIH_LAUNCH(kWave, 4);
+        if (w == 7) DCIH_LAUNCH_COMPACT(7); else if (w == 6) DCIH_LAUNCH_COMPACT(6);
+        else if (w == 5) DCIH_LAUNCH_COMPACT(5); else DCIH_LAUNCH_COMPACT(4);
         DCIH_HIP(hipGetLastError());
         return 0;
     }
@@ -1215,6 +1232,8 @@ static int launch_block(const QueryArgs& a, const BlockLayout& y, int64_t items,
         else DCIH_LAUNCH(kBlockThreads, 3);
     }
 #undef DCIH_LAUNCH
+#undef DCIH_LAUNCH_COMPACT
+#undef DCIH_LAUNCH_KERNEL
     DCIH_HIP(hipGetLastError());
     return 0;
 }
