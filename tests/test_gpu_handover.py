@@ -79,3 +79,38 @@ def test_items_handed_to_the_dense_kernel_answer_alike(gpu, oracle, shape):
     assert t_batch >= 0.0
     assert torch.equal(got[0], want[0]) and torch.equal(got[1], want[1])
     dci.free()
+
+
+def test_items_that_outgrow_the_compact_tables_answer_alike(gpu, oracle):
+    """The batch kernel's one-wavefront variants keep an item's flags in a small hashed set; an
+    item that promotes more points than the set takes is listed and computed again by the
+    variant with the full tables.  The phase profile counts the items handed back: some must
+    be (the premise), and ids, distances and counters must not show it."""
+    from dciknn_cuda_amd import _capi
+    n, dim, M, L, B, T, k, outer, nq = 60_000, 16, 2, 10, 3, 4, 15, 100, 96
+    rng = np.random.default_rng(5)
+    X = rng.standard_normal((n, dim)).astype(np.float32)
+    Q = rng.standard_normal((nq, dim)).astype(np.float32)
+    dci = gpu.DCI(dim, M, L, B, T, seed=9, traversal="batch")
+    lib, h = dci._lib, dci._dci_inst
+    dci.add(torch.from_numpy(X).cuda())
+    skeys, sids = engine_index(dci)
+    qproj = engine_project(dci.directions.numpy(), Q).T.copy()
+    ref = oracle.query(skeys, sids, X, Q, qproj, M, L, B, T, k, outer, max_cand=10 * k)
+    rc = ref["counters"].astype(np.int64)
+    qd = torch.from_numpy(Q).cuda()
+    ticks = torch.zeros(16, dtype=torch.int64, device="cuda")
+    _capi.check(lib.dcih_phase_profile(h, ticks.data_ptr()))
+    for call in range(2):       # the second call routes by the recorded stops as well
+        ids, dists, ctr = dci.query(qd, k, outer, return_int=True, return_counters=True)
+        torch.cuda.synchronize()
+        ids, dists, ctr = ids.cpu().numpy(), dists.cpu().numpy(), ctr.cpu().numpy().astype(np.int64)
+        np.testing.assert_array_equal(ids, ref["ids"])
+        np.testing.assert_allclose(dists, ref["dists"], rtol=1e-5, atol=1e-6)
+        np.testing.assert_array_equal(ctr[:, 1], rc[:, 1])
+        np.testing.assert_array_equal(ctr[:, 3], rc[:, 3])
+    _capi.check(lib.dcih_phase_profile(h, None))
+    t = ticks.cpu().numpy()
+    assert t[10] > 0, "no item was handed from the compact tables to the second pass"
+    assert t[9] == 2 * nq * B, (t[9], "every item finished in the batch kernel, first or second pass")
+    dci.free()

@@ -224,7 +224,7 @@ CASES = [
     (3000, 8, 1100, 2, 4, 3, 16, 10, 5, "normal"),          # long rows: five pieces, the last one short
     (120000, 8, 16, 3, 16, 2, 8, 10, 30, "normal"),         # 60000-point partitions, 48 indices: the step kernel's counters leave LDS, the batch kernel's flags do not
     (60000, 48, 16, 2, 10, 3, 2, 10, 100, "normal"),        # the batch kernel's compact tables, two-stage scan; one wavefront per item
-    (60000, 48, 16, 2, 10, 3, 4, 30, 100, "normal"),        # ... with items that outgrow them and go to its second pass
+    (60000, 48, 16, 2, 10, 3, 4, 15, 100, "normal"),        # ... with items that outgrow them and go to its second pass
     (64000, 16, 8, 26, 1, 1, 2, 10, 5, "normal"),           # compact tables, 26 composites: the full tables would not fit LDS (no second pass)
 ]
 
