@@ -705,9 +705,9 @@ __device__ __forceinline__ void traverse_block_item(const QueryArgs& a, const Bl
         }
         PHASE_FENCE();
         {
-            // Eight lanes rank one promotion, so 32 promotions are in flight per
-            // workgroup; each lane runs the binary searches of up to three streams in
-            // lockstep so that their key reads overlap.
+            // Four lanes rank one promotion, so 16 promotions are in flight per wavefront;
+            // each lane runs the binary searches of up to five streams in lockstep so that
+            // their key reads overlap.
             constexpr int kGroup = 4, kPerLane = 5;
             const int gl = tid & (kGroup - 1);
             const int group = tid / kGroup;
