@@ -18,7 +18,9 @@ extern "C" {
  * reference).  d_ticks is NULL (off) or a zeroed device array of 16 uint64 that
  * later dcih_query calls add to: [0..7] = 100 MHz ticks one thread of every
  * workgroup spent in set-up, bound selection, range search, streaming, undo,
- * promotion ranking, replay, distances/top-k; [8] = epochs, [9] = workgroups.
+ * promotion ranking, replay, distances/top-k; [8] = epochs, [9] = items finished by
+ * the batch kernel (either pass), [10] = items it handed back (to its second pass with
+ * the full tables, or to the step-by-step kernel), [11..14] = those by reason.
  */
 int dcih_phase_profile(dcih_index* h, uint64_t* d_ticks);
 
